@@ -26,7 +26,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..parts.base import PagedKVSpec, StateSpec
+from ..parts.base import PagedKVSpec, StateSpec, paged_part, state_part
 from .pages import CacheExhaustedError, CacheStateError, PagePool
 
 
@@ -116,12 +116,13 @@ class CacheManager:
         self.state_specs: Dict[int, StateSpec] = {}
         by_spec: Dict[PagedKVSpec, List[int]] = {}
         for cache, spec in sorted(cache_specs.items()):
-            if isinstance(spec, PagedKVSpec):
-                by_spec.setdefault(spec, []).append(cache)
-            elif isinstance(spec, StateSpec):
-                self.state_specs[cache] = spec
-            else:
+            paged, state = paged_part(spec), state_part(spec)
+            if paged is None and state is None:
                 raise TypeError(f"cache {cache}: unknown cache spec {spec!r}")
+            if paged is not None:
+                by_spec.setdefault(paged, []).append(cache)
+            if state is not None:
+                self.state_specs[cache] = state
         for spec, caches in by_spec.items():
             pages = num_pages[len(self.groups)] if isinstance(num_pages, (list, tuple)) else num_pages
             group = CacheGroup(len(self.groups), spec, caches, pages, page_size)
@@ -151,7 +152,7 @@ class CacheManager:
     @staticmethod
     def bytes_per_token(cache_specs: Dict[int, object], dtype: torch.dtype) -> int:
         size = torch.empty(0, dtype=dtype).element_size()
-        return sum(2 * spec.n_kv_heads * spec.head_dim * size for spec in cache_specs.values() if isinstance(spec, PagedKVSpec))
+        return sum(2 * spec.n_kv_heads * spec.head_dim * size for spec in map(paged_part, cache_specs.values()) if spec is not None)
 
     # -- views for the model ---------------------------------------------------------------
     def view(self, call) -> LayerCacheView:
@@ -160,7 +161,8 @@ class CacheManager:
             group = self.groups[self.group_of_cache[cache]]
             layer = self.layer_in_group[cache]
             return LayerCacheView(group.index, None if group.keys is None else group.keys[layer],
-                                  None if group.values is None else group.values[layer], self.page_size, call.writes_cache)
+                                  None if group.values is None else group.values[layer], self.page_size, call.writes_cache,
+                                  self.state.get(cache))
         if cache in self.state:
             return LayerCacheView(-1, None, None, self.page_size, call.writes_cache, self.state[cache])
         return LayerCacheView(-1, None, None, self.page_size, call.writes_cache)

@@ -37,9 +37,9 @@ def resolve_architecture(name: str) -> Tuple[Type[ModelConfig], Callable]:
 
 
 def config_from_dict(raw: dict) -> ModelConfig:
-    name = raw.get("model_type")
+    name = raw.get("model_type", raw.get("architecture"))         # (either key may name it)
     if not isinstance(name, str):
-        raise UnsupportedModelError("config.json has no 'model_type' string naming the architecture")
+        raise UnsupportedModelError("config.json has no 'model_type' (or 'architecture') string naming the architecture")
     config_class, _ = resolve_architecture(name)
     return config_class.from_dict(raw)
 

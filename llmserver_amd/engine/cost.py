@@ -13,7 +13,7 @@ from typing import Dict, Iterable, Sequence
 
 import torch
 
-from ..parts.base import MATRIX, PagedKVSpec, ParamSpec, StateSpec
+from ..parts.base import MATRIX, ParamSpec, paged_part, state_part
 
 
 @dataclasses.dataclass(frozen=True)
@@ -62,12 +62,13 @@ def cache_bytes(model, rows: Sequence[StepRow], dtype: torch.dtype) -> float:
     element = torch.empty((), dtype=dtype).element_size()
     total = 0.0
     for call in model.order:
-        spec = model.blocks[call.block].mixer.cache_spec()
-        if isinstance(spec, PagedKVSpec):
+        whole = model.blocks[call.block].cache_spec()
+        spec, state = paged_part(whole), state_part(whole)
+        if spec is not None:
             keys = sum(min(row.context, spec.window) if spec.window else row.context for row in rows)
             total += 2.0 * spec.n_kv_heads * spec.head_dim * element * keys
-        elif isinstance(spec, StateSpec):
-            total += math.prod(spec.shape) * torch.empty((), dtype=getattr(torch, spec.dtype)).element_size() * len(rows)
+        if state is not None:
+            total += math.prod(state.shape) * torch.empty((), dtype=getattr(torch, state.dtype)).element_size() * len(rows)
     return total
 
 

@@ -26,6 +26,7 @@ from datetime import datetime, timedelta
 from typing import Dict, List, Optional
 
 from ..cache import CacheExhaustedError, CacheManager
+from ..parts.base import paged_part
 from ..sampling import Sampler, request_uniform
 from .batch import StepEntry
 from .request import CompletedRequest, Request, RequestFinishReason, RequestStatus, SamplingParams
@@ -332,7 +333,7 @@ class Engine:
         tiles (the step's plan then gives every tile a wavefront of its own, which reads its keys itself: correct,
         and about half as fast on long prompts)."""
         import warnings
-        for head_dim in sorted({spec.head_dim for spec in model.cache_specs().values() if hasattr(spec, "head_dim")}):
+        for head_dim in sorted({paged.head_dim for paged in map(paged_part, model.cache_specs().values()) if paged is not None}):
             if ops.attention_workgroup_tiles(self.dtype, head_dim) and not ops.attention_workgroup_tiles(self.dtype, head_dim, page_size):
                 warnings.warn(f"kv_cache_block_size={page_size}: the attention kernel for prompt portions takes pages of a multiple of 8 keys "
                               f"in {str(self.dtype).split('.')[-1]}; with this page size prompts run through the slower per-tile kernel "

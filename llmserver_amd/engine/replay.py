@@ -21,6 +21,7 @@ from typing import Iterable, TextIO
 import torch
 
 from ..cache import CacheManager
+from ..parts.base import paged_part
 from .batch import StepEntry
 from .loading import load_model, parse_dtype
 from .step import ModelRunner
@@ -37,7 +38,7 @@ def make_runner(model_dir: str, dtype, max_tokens: int, page_size: int = 16, dev
         from ..kernels import default_ops
         ops = default_ops()
     specs = model.cache_specs()
-    head_dims = sorted({spec.head_dim for spec in specs.values() if hasattr(spec, "head_dim")})
+    head_dims = sorted({paged.head_dim for paged in map(paged_part, specs.values()) if paged is not None})
     ops.preload(head_dims, dtype)
     pages = max(1, -(-max_tokens // page_size))
     cache = CacheManager(specs, page_size, pages, num_state_slots=max_live, device=model.device, dtype=dtype,

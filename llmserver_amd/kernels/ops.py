@@ -14,6 +14,7 @@ import dataclasses
 import torch
 
 from ..parts.attention import AttentionTuning, TileLaunchCost, group_tiling
+from ..parts.base import paged_part
 from ..parts.kernel_namespace import KernelNamespace
 from . import build, library
 from .choices import ChoiceTable, choice_key
@@ -144,9 +145,9 @@ class HipOps(KernelNamespace):
                 raise ValueError(f"a pool of {most} pages of {page_size} keys lets a context reach {most * page_size} keys; the attention "
                                  f"kernels find a key's page exactly only below 2^32 / page_size = {(1 << 32) // page_size} keys")
         for spec in cache_specs.values():
-            head_dim = getattr(spec, "head_dim", None)
-            if head_dim is not None:
-                build.attention_module(True, head_dim)      # raises with the sizes the kernels take
+            paged = paged_part(spec)
+            if paged is not None:
+                build.attention_module(True, paged.head_dim)      # raises with the sizes the kernels take
 
     @staticmethod
     def required_modules(head_dims, dtype):

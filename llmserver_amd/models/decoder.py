@@ -25,10 +25,18 @@ class LayerCall:
     writes_cache: bool = True   # False: read the cache another call has written
 
 
+def joined(prefix: str, name: str) -> str:
+    """``prefix.name``, or the prefix alone for a part whose own name is its tensor's."""
+    return f"{prefix}.{name}" if name else prefix
+
+
 class DecoderModel:
+    """``names``: the checkpoint's names of the embedding, of the list of layers and of the final norm; layer ``i``'s
+    tensors start with ``layer_name(i)`` (default: ``<layers>.<i>``)."""
+
     def __init__(self, config, embedding: TokenEmbedding, blocks: Sequence[Block], final_norm: Norm, head: Linear,
                  tie_head: bool, order: Optional[Sequence[LayerCall]] = None,
-                 names=("model.embed_tokens", "model.layers", "model.norm")):
+                 names=("model.embed_tokens", "model.layers", "model.norm"), layer_name=None):
         self.config = config
         self.embedding = embedding
         self.blocks = list(blocks)
@@ -37,6 +45,8 @@ class DecoderModel:
         self.tie_head = tie_head
         self.order = list(order) if order is not None else [LayerCall(i, i) for i in range(len(self.blocks))]
         self.embed_name, self.layers_name, self.norm_name = names
+        self.layer_name = layer_name if layer_name is not None else (lambda index: f"{self.layers_name}.{index}")
+        self._owners = None
         self.device = None
         self.dtype = None
         self._check_order()
@@ -52,49 +62,52 @@ class DecoderModel:
                     raise ValueError(f"cache {call.cache} is written by two calls of the order")
                 writers[call.cache] = call.block
         for call in self.order:
-            spec = self.blocks[call.block].mixer.cache_spec()
+            spec = self.blocks[call.block].cache_spec()
             if spec is None:
                 continue
             if call.cache not in writers:
                 raise ValueError(f"cache {call.cache} is read but never written")
-            if self.blocks[writers[call.cache]].mixer.cache_spec() != spec:
+            if self.blocks[writers[call.cache]].cache_spec() != spec:
                 raise ValueError(f"cache {call.cache} is shared by mixers with different cache needs")
 
     def cache_specs(self) -> Dict[int, object]:
         """cache index -> what its writer stores."""
         specs = {}
         for call in self.order:
-            spec = self.blocks[call.block].mixer.cache_spec()
+            spec = self.blocks[call.block].cache_spec()
             if spec is not None and call.writes_cache:
                 specs[call.cache] = spec
         return specs
 
     # -- parameters --------------------------------------------------------------------
-    def param_specs(self) -> Dict[str, ParamSpec]:
-        specs = {f"{self.embed_name}.{k}": v for k, v in self.embedding.param_specs().items()}
+    def _named(self):
+        """(checkpoint name, owning part, the part's own name of the tensor, spec) of every tensor."""
+        for k, v in self.embedding.param_specs().items():
+            yield joined(self.embed_name, k), self.embedding, k, v
         for i, block in enumerate(self.blocks):
-            specs.update({f"{self.layers_name}.{i}.{k}": v for k, v in block.param_specs().items()})
-        specs.update({f"{self.norm_name}.{k}": v for k, v in self.final_norm.param_specs().items()})
+            for k, v in block.param_specs().items():
+                yield joined(self.layer_name(i), k), block, k, v
+        for k, v in self.final_norm.param_specs().items():
+            yield joined(self.norm_name, k), self.final_norm, k, v
         for k, v in self.head.param_specs().items():
             # Tied when the configuration says so or the checkpoint holds no head
             # (utils/model_loader.py:56-59).
-            specs[k] = dataclasses.replace(v, optional=True)
-        return specs
+            yield k, self.head, k, dataclasses.replace(v, optional=True)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {name: spec for name, _, _, spec in self._named()}
 
     def ignored_names(self):
         """Checkpoint tensors that may be present but are not read."""
         return set(self.head.param_specs()) if self.tie_head else set()
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
-        if name.startswith(self.embed_name + "."):
-            self.embedding.assign(name[len(self.embed_name) + 1:], tensor)
-        elif name.startswith(self.layers_name + "."):
-            index, rest = name[len(self.layers_name) + 1:].split(".", 1)
-            self.blocks[int(index)].assign(rest, tensor)
-        elif name.startswith(self.norm_name + "."):
-            self.final_norm.assign(name[len(self.norm_name) + 1:], tensor)
-        else:
-            self.head.assign(name, tensor)
+        if self._owners is None:
+            self._owners = {full: (part, own) for full, part, own, _ in self._named()}
+        if name not in self._owners:
+            raise KeyError(name)
+        part, own = self._owners[name]
+        part.assign(own, tensor)
 
     def finalize(self, assigned: Sequence[str], device, dtype) -> None:
         head_names = set(self.head.param_specs())

@@ -1,15 +1,19 @@
 from .attention import AttentionNames, AttentionPlan, AttentionTuning, GQAttention, TileLaunchCost, build_attention_plan, group_tiling
-from .base import (INT_TABLE, MATRIX, VECTOR, Block, FeedForward, Mixer, Norm, PagedKVSpec, ParamSpec, Part,
+from .base import (INT_TABLE, MATRIX, VECTOR, Block, FeedForward, Mixer, Norm, PagedAndStateSpec, PagedKVSpec, ParamSpec, Part,
                    PositionEncoding, StateSpec)
-from .block import PreNormBlock
-from .embedding import TokenEmbedding
+from .block import DepthAverage, PostNormBlock, PreNormBlock
+from .conv import ShortConvolution
+from .embedding import NormedTokenEmbedding, TokenEmbedding
+from .experts import RoutedExperts
 from .kernel_namespace import KernelNamespace
+from .latent_attention import LatentAttention, LatentAttentionNames
 from .linear import Linear
 from .mlp import GatedMLP, GatedMLPNames
 from .norm import RMSNorm
-from .rope import NoPosition, RotaryPosition
+from .rope import NoPosition, PairedRotaryPosition, RotaryPosition
 
 __all__ = ["KernelNamespace", "AttentionNames", "AttentionTuning", "TileLaunchCost", "GatedMLPNames", "AttentionPlan", "GQAttention", "build_attention_plan", "group_tiling", "INT_TABLE", "MATRIX", "VECTOR",
            "Block", "FeedForward", "Mixer", "Norm", "PagedKVSpec", "ParamSpec", "Part", "PositionEncoding",
            "StateSpec", "PreNormBlock", "TokenEmbedding", "Linear", "GatedMLP", "RMSNorm", "NoPosition",
-           "RotaryPosition"]
+           "RotaryPosition", "PairedRotaryPosition", "PagedAndStateSpec", "DepthAverage", "PostNormBlock", "ShortConvolution",
+           "NormedTokenEmbedding", "RoutedExperts", "LatentAttention", "LatentAttentionNames"]

@@ -392,6 +392,55 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     return plan
 
 
+def stage_attention_plan(ctx, key, group_size: int, n_kv_heads: int, head_dim: int, window: Optional[int], graph_shape) -> None:
+    """Make the step's attention work list for a mixer of this geometry and put it among the step's staged arrays under
+    ``key`` (mixers of equal geometry share it).  ``graph_shape``: the mixer's :meth:`Mixer.graph_shape`."""
+    if ctx.has_plan(key):
+        return
+    fixed = fixed_tiles = None
+    tuning = tuning_of(ctx.ops, DEFAULT_TUNING, ctx.dtype, head_dim)
+    single_tokens = ctx.n_tokens == ctx.n_rows
+    if ctx.static_max_keys is not None and single_tokens:          # a step whose shapes must not depend on the contexts
+        fixed = fixed_split_count(ctx.n_rows, group_size, n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
+    elif ctx.static_max_keys is not None:
+        # ... nor on how its tokens are spread over its rows: as many tiles as rows of this many tokens can have at
+        # most (a row's last tile may be partly empty), every tile with the same number of key ranges.
+        _, tokens_per_tile, _ = group_tiling(group_size, tuning.tile_rows)
+        fixed_tiles = ctx.n_tokens // tokens_per_tile + ctx.n_rows
+        fixed = fixed_split_count(fixed_tiles, group_size, n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
+    # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
+    #  * short contexts (a shape of captured steps of its own, see graph_shape): four ranges a tile, in steps of
+    #    single tokens and in captured steps with portions alike;
+    #  * so many rows that a tile gets four ranges anyway;
+    #  * two ranges a tile: two tiles to a workgroup, if the rows come in pairs.  (Two or three ranges in a workgroup
+    #    of one tile leave wavefronts idle through the others' walk: a tenth slower at 64 rows behind 4,096 tokens.)
+    in_workgroup = 0
+    if single_tokens:
+        if ctx.static_max_keys is not None and graph_shape(ctx.n_rows, int(np.max(ctx.h_row_ctx))) is not None:
+            in_workgroup = fixed = WORKGROUP_RANGES
+        elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
+            in_workgroup = fixed
+    elif ctx.static_max_keys is not None and graph_shape(ctx.n_rows, int(np.max(ctx.h_row_ctx))) is not None:
+        in_workgroup = fixed = WORKGROUP_RANGES
+    per_workgroup = ctx.ops.attention_workgroup_tiles(ctx.dtype, head_dim, ctx.page_size)
+    halves = ctx.ops.attention_tile_halves(ctx.dtype, head_dim) if per_workgroup else 1
+    fewest = ctx.ops.attention_tile_min_workgroups(ctx.dtype) if per_workgroup else 0
+    key_ranges = ctx.ops.attention_tile_key_ranges(ctx.dtype, head_dim) if per_workgroup else 1
+    plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, group_size, n_kv_heads, window,
+                                target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
+                                merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves, tile_min_workgroups=fewest,
+                                tile_key_ranges=key_ranges, fixed_tiles=fixed_tiles)
+    ctx.set_plan(key, {
+        **({"tile_slots": plan.tile_slots} if plan.tile_slots is not None else {}),
+        "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
+        "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
+        "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup, "tile_halves": int(plan.tile_halves),
+        "merge_in_workgroup": int(plan.merge_in_workgroup),
+        "most_splits": int(plan.merges[:, 3].max()) if len(plan.merges) else 0,
+    })
+
+
+
 class GQAttention(Mixer):
     graph_safe = True
     accepts_pending_norm = True
@@ -399,7 +448,10 @@ class GQAttention(Mixer):
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
-                 window: Optional[int] = None, scale: Optional[float] = None, names: AttentionNames = AttentionNames()):
+                 window: Optional[int] = None, scale: Optional[float] = None, names: AttentionNames = AttentionNames(),
+                 sinks: Optional[str] = None):
+        """``sinks``: the checkpoint name of a float vector ``[n_heads]`` whose exponentials join the softmax's
+        denominators (one term per head, without a key or a value), or None."""
         if n_heads % n_kv_heads:
             raise ValueError(f"Number of query heads must be divisible by the number of KV heads: query heads: {n_heads}, KV heads: {n_kv_heads}")
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
@@ -420,6 +472,7 @@ class GQAttention(Mixer):
         self.o = Linear(q_rows, (names.out,), (width,), bias if out_bias is None else out_bias)
         self.q_norm_weight = None
         self.k_norm_weight = None
+        self.sinks_name, self.sinks = sinks, None
 
     def cache_spec(self):
         return PagedKVSpec(self.n_kv_heads, self.head_dim, self.window)
@@ -429,11 +482,15 @@ class GQAttention(Mixer):
         if self.qk_norm_eps is not None:
             specs[f"{self.names.q_norm}.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
             specs[f"{self.names.k_norm}.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
+        if self.sinks_name is not None:
+            specs[self.sinks_name] = ParamSpec((self.n_heads,), VECTOR, "normal")
         return specs
 
     def assign(self, name, tensor):
         owner = name.rsplit(".", 1)[0]
-        if owner == self.names.q_norm:
+        if name == self.sinks_name:
+            self.sinks = tensor
+        elif owner == self.names.q_norm:
             self.q_norm_weight = tensor
         elif owner == self.names.k_norm:
             self.k_norm_weight = tensor
@@ -467,50 +524,7 @@ class GQAttention(Mixer):
         return 4.0 * self.n_heads * self.head_dim * pairs
 
     def prepare(self, ctx):
-        key = self.plan_key()
-        if ctx.has_plan(key):
-            return
-        fixed = fixed_tiles = None
-        tuning = tuning_of(ctx.ops, DEFAULT_TUNING, ctx.dtype, self.head_dim)
-        single_tokens = ctx.n_tokens == ctx.n_rows
-        if ctx.static_max_keys is not None and single_tokens:          # a step whose shapes must not depend on the contexts
-            fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
-        elif ctx.static_max_keys is not None:
-            # ... nor on how its tokens are spread over its rows: as many tiles as rows of this many tokens can have at
-            # most (a row's last tile may be partly empty), every tile with the same number of key ranges.
-            _, tokens_per_tile, _ = group_tiling(self.group_size, tuning.tile_rows)
-            fixed_tiles = ctx.n_tokens // tokens_per_tile + ctx.n_rows
-            fixed = fixed_split_count(fixed_tiles, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
-        # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
-        #  * short contexts (a shape of captured steps of its own, see graph_shape): four ranges a tile, in steps of
-        #    single tokens and in captured steps with portions alike;
-        #  * so many rows that a tile gets four ranges anyway;
-        #  * two ranges a tile: two tiles to a workgroup, if the rows come in pairs.  (Two or three ranges in a workgroup
-        #    of one tile leave wavefronts idle through the others' walk: a tenth slower at 64 rows behind 4,096 tokens.)
-        in_workgroup = 0
-        if single_tokens:
-            if ctx.static_max_keys is not None and self.graph_shape(ctx.n_rows, int(np.max(ctx.h_row_ctx))) is not None:
-                in_workgroup = fixed = WORKGROUP_RANGES
-            elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
-                in_workgroup = fixed
-        elif ctx.static_max_keys is not None and self.graph_shape(ctx.n_rows, int(np.max(ctx.h_row_ctx))) is not None:
-            in_workgroup = fixed = WORKGROUP_RANGES
-        per_workgroup = ctx.ops.attention_workgroup_tiles(ctx.dtype, self.head_dim, ctx.page_size)
-        halves = ctx.ops.attention_tile_halves(ctx.dtype, self.head_dim) if per_workgroup else 1
-        fewest = ctx.ops.attention_tile_min_workgroups(ctx.dtype) if per_workgroup else 0
-        key_ranges = ctx.ops.attention_tile_key_ranges(ctx.dtype, self.head_dim) if per_workgroup else 1
-        plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
-                                    target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
-                                    merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves, tile_min_workgroups=fewest,
-                                    tile_key_ranges=key_ranges, fixed_tiles=fixed_tiles)
-        ctx.set_plan(key, {
-            **({"tile_slots": plan.tile_slots} if plan.tile_slots is not None else {}),
-            "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
-            "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
-            "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup, "tile_halves": int(plan.tile_halves),
-            "merge_in_workgroup": int(plan.merge_in_workgroup),
-            "most_splits": int(plan.merges[:, 3].max()) if len(plan.merges) else 0,
-        })
+        stage_attention_plan(ctx, self.plan_key(), self.group_size, self.n_kv_heads, self.head_dim, self.window, self.graph_shape)
 
     def forward(self, x, ctx, cache, sink=None):
         qkv = self.qkv.forward(x, ctx)
@@ -530,6 +544,8 @@ class GQAttention(Mixer):
                 cos_sin, cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim, cache.writable)
         out = ctx.empty((qkv.shape[0], self.n_heads * self.head_dim))
         extra = {"decode_fusion": fusion} if fusion is not None else {}
+        if self.sinks is not None:
+            extra["sinks"] = self.sinks
         ctx.ops.paged_attention(
             qkv, out, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
             ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size,

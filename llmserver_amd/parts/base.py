@@ -48,6 +48,29 @@ class StateSpec:
     dtype: str = "float32"
 
 
+@dataclasses.dataclass(frozen=True)
+class PagedAndStateSpec:
+    """Pages of keys and values and, beside them, a state of fixed size per request: what a layer call needs whose
+    mixer attends over a paged cache while another part of the block (a short convolution in front of the mixer,
+    say) carries a few rows from one step to the next."""
+    paged: PagedKVSpec
+    state: StateSpec
+
+
+def paged_part(spec) -> Optional[PagedKVSpec]:
+    """The paged share of a cache spec, or None."""
+    if isinstance(spec, PagedKVSpec):
+        return spec
+    return spec.paged if isinstance(spec, PagedAndStateSpec) else None
+
+
+def state_part(spec) -> Optional[StateSpec]:
+    """The per-request state of a cache spec, or None."""
+    if isinstance(spec, StateSpec):
+        return spec
+    return spec.state if isinstance(spec, PagedAndStateSpec) else None
+
+
 class Part:
     """Common base: named tensors in, nothing model-specific."""
 
@@ -173,7 +196,7 @@ class Mixer(Part):
     takes_sink = False
 
     def cache_spec(self):
-        """:class:`PagedKVSpec`, :class:`StateSpec` or None."""
+        """:class:`PagedKVSpec`, :class:`StateSpec`, :class:`PagedAndStateSpec` or None."""
         return None
 
     def prepare(self, ctx) -> None:
@@ -222,6 +245,10 @@ class Block(Part):
     def entry_norm(self):
         """The norm this block applies first to what it is given, or None."""
         return None
+
+    def cache_spec(self):
+        """What a call of this block keeps between steps: the mixer's needs, unless the block adds its own."""
+        return self.mixer.cache_spec()
 
     def forward(self, resid, delta, ctx, cache):
         raise NotImplementedError

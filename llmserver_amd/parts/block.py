@@ -6,7 +6,10 @@ is still to be added travel as a pair, so every "add, then normalise" is one ker
 """
 from __future__ import annotations
 
-from .base import Block, FeedForward, Mixer, Norm, ResidualSink, StreamUpdate
+import torch
+
+from .base import (VECTOR, Block, FeedForward, Mixer, Norm, PagedAndStateSpec, PagedKVSpec, ParamSpec, Part, ResidualSink,
+                   StreamUpdate)
 
 
 class PreNormBlock(Block):
@@ -60,3 +63,118 @@ class PreNormBlock(Block):
         """``following``: the norm that will be applied to this block's output, if the caller knows it."""
         resid, mixed = self._feed(self.mixer_norm, self.mixer, resid, delta, ctx, cache, following=self.ffn_norm)
         return self._feed(self.ffn_norm, self.ffn, resid, mixed, ctx, following=following)
+
+
+class DepthAverage(Part):
+    """What a layer hands on is a weighted sum of the embedding's output and the results of all layers so far:
+    ``sum_{j <= i + 1} w[j] * X_j`` behind layer ``i`` (``X_0`` the embedding's output, ``X_(j+1)`` layer ``j``'s own
+    result).  The results of a step's tokens are kept for the length of the step, in 32-bit; ``states`` is how many a
+    model has (its layers and one).  Layer ``i``'s weights are a vector of ``i + 2`` numbers."""
+
+    def __init__(self, index: int, states: int, tensor: str = "dwa"):
+        self.index, self.states, self.tensor = index, states, tensor
+        self.weights = None     # float32 [index + 2]
+
+    def param_specs(self):
+        return {self.tensor: ParamSpec((self.index + 2,), VECTOR, "norm")}
+
+    def assign(self, name, tensor):
+        assert name == self.tensor
+        self.weights = tensor
+
+    def history(self, x, ctx):
+        """The step's kept results ``[states, T, W]``; the first layer puts the embedding's output there."""
+        kept = ctx.computed(("depth average", self.states), lambda: ctx.empty((self.states, *x.shape), dtype=torch.float32))
+        if self.index == 0:
+            kept[0].copy_(x)
+        return kept
+
+
+class PostNormBlock(Block):
+    """Sublayers that read the stream itself and are normalised on their way out:
+    ``x <- x + s1 * n1(mixer(x + conv(x)))``, then ``x <- x + s2 * n2(ffn(x))``, the stream in 32-bit throughout.
+
+    ``conv`` (a :class:`~llmserver_amd.parts.conv.ShortConvolution` or None) stands in front of the mixer and keeps a
+    per-request state beside the mixer's cache; ``scales`` says whether per-channel scales ``ls1`` / ``ls2`` multiply the
+    normalised results; ``ffn`` may be None; ``average`` (a :class:`DepthAverage` or None) mixes the layer's result with
+    the results before it.  The sum, the norm, the scale and the average behind a sublayer are one kernel."""
+
+    def __init__(self, mixer: Mixer, mixer_norm: Norm, ffn, ffn_norm, conv=None, scales: bool = True, average=None,
+                 names=("mix", "norm1", "mlp", "norm2", "canon1", "ls1", "ls2")):
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm, self.conv, self.average = mixer, mixer_norm, ffn, ffn_norm, conv, average
+        self.names = tuple(names)
+        self.scales = scales
+        self.scale1 = self.scale2 = None
+        self.width = mixer_norm.width
+
+    def _parts(self):
+        mix, norm1, mlp, norm2, conv = self.names[:5]
+        parts = {mix: self.mixer, norm1: self.mixer_norm}
+        if self.ffn is not None:
+            parts.update({mlp: self.ffn, norm2: self.ffn_norm})
+        if self.conv is not None:
+            parts[conv] = self.conv
+        return parts
+
+    def param_specs(self):
+        specs = {f"{prefix}.{name}" if name else prefix: spec for prefix, part in self._parts().items()
+                 for name, spec in part.param_specs().items()}
+        if self.scales:
+            specs[self.names[5]] = ParamSpec((self.width,), VECTOR, "norm")
+            if self.ffn is not None:
+                specs[self.names[6]] = ParamSpec((self.width,), VECTOR, "norm")
+        if self.average is not None:
+            specs.update(self.average.param_specs())
+        return specs
+
+    def assign(self, name, tensor):
+        if self.scales and name in self.names[5:7]:
+            if name == self.names[5]:
+                self.scale1 = tensor
+            else:
+                self.scale2 = tensor
+            return
+        if self.average is not None and name in self.average.param_specs():
+            self.average.assign(name, tensor)
+            return
+        parts = self._parts()
+        if name in parts:                                   # the part's name is the tensor's
+            parts[name].assign("", tensor)
+            return
+        prefix, rest = name.split(".", 1)
+        parts[prefix].assign(rest, tensor)
+
+    def finalize(self):
+        for part in self._parts().values():
+            part.finalize()
+
+    def cache_spec(self):
+        spec = self.mixer.cache_spec()
+        state = self.conv.state_spec() if self.conv is not None else None
+        if state is None:
+            return spec
+        if not isinstance(spec, PagedKVSpec):
+            raise ValueError("a convolution in front of the mixer keeps its state beside a paged cache only")
+        return PagedAndStateSpec(spec, state)
+
+    def forward(self, resid, delta, ctx, cache):
+        if delta is not None:
+            raise ValueError("this block takes a stream to which everything has been added")
+        x = resid
+        ops = ctx.ops
+        wide = ctx.dtype == torch.float32
+        h = self.conv.forward(x, ctx, cache.state) if self.conv is not None else (x if wide else x.to(ctx.dtype))
+        mixed = self.mixer.forward(h, ctx, cache)
+        last = self.ffn is None
+        history = self.average.history(x, ctx) if self.average is not None else None
+        after = {"history": history, "before": self.average.index + 1, "mix": self.average.weights} if history is not None else {}
+        out = ctx.empty(x.shape, dtype=torch.float32)
+        if last:
+            ops.scaled_norm_add(x, mixed, self.mixer_norm.weight, self.scale1, self.mixer_norm.eps, out, **after)
+            return out, None
+        rounded = None if wide else ctx.empty(x.shape)
+        ops.scaled_norm_add(x, mixed, self.mixer_norm.weight, self.scale1, self.mixer_norm.eps, out, rounded=rounded)
+        fed = self.ffn.forward(out if wide else rounded, ctx)
+        result = ctx.empty(x.shape, dtype=torch.float32)
+        ops.scaled_norm_add(out, fed, self.ffn_norm.weight, self.scale2, self.ffn_norm.eps, result, **after)
+        return result, None

@@ -1,6 +1,8 @@
 """Token embedding lookup ``h0 = E[ids]`` without scaling (utils/model.py:56-59,110)."""
 from __future__ import annotations
 
+import torch
+
 from .base import MATRIX, ParamSpec, Part
 
 
@@ -19,4 +21,33 @@ class TokenEmbedding(Part):
     def forward(self, token_ids, ctx):
         out = ctx.empty((token_ids.shape[0], self.width))
         ctx.ops.embedding(self.weight, token_ids, out)
+        return out
+
+
+class NormedTokenEmbedding(Part):
+    """Lookup followed by a norm, as one kernel, into a 32-bit residual stream: ``x = norm(E[ids])``.  The table's
+    tensor has the part's own name, the norm's weight the name ``norm`` below it."""
+
+    def __init__(self, vocab: int, width: int, norm, table: str = "", norm_name: str = "norm"):
+        self.vocab, self.width, self.norm = vocab, width, norm
+        self.table_name, self.norm_name = table, norm_name
+        self.weight = None
+
+    def param_specs(self):
+        specs = {self.table_name: ParamSpec((self.vocab, self.width), MATRIX, "normal", share_per_token=0.0)}
+        for name, spec in self.norm.param_specs().items():
+            specs[f"{self.norm_name}.{name}" if name else self.norm_name] = spec
+        return specs
+
+    def assign(self, name, tensor):
+        if name == self.table_name:
+            self.weight = tensor
+        elif name == self.norm_name:
+            self.norm.assign("", tensor)
+        else:
+            self.norm.assign(name[len(self.norm_name) + 1:], tensor)
+
+    def forward(self, token_ids, ctx):
+        out = ctx.empty((token_ids.shape[0], self.width), dtype=torch.float32)
+        ctx.ops.embedding_norm(self.weight, token_ids, self.norm.weight, self.norm.eps, out)
         return out

@@ -1,0 +1,65 @@
+"""Routed experts: every token's feed-forward is a weighted sum of ``top`` of ``experts`` small gated feed-forwards.
+
+Router logits ``z = R h`` in 32-bit; the ``top`` largest are chosen (the first of equal ones) and weighted by the softmax
+over the chosen logits only.  Expert: ``D (act(G h) * (U h))`` with ``act = silu``; no biases.  The experts' matrices
+are stacked (``[experts, 2F, W]`` gate rows then up rows, ``[experts, W, F]``), and the kernels pick each token's from
+the list of chosen experts on the device: nothing of the routing is read on the host.
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import VECTOR, FeedForward, ParamSpec
+
+
+class RoutedExperts(FeedForward):
+    def __init__(self, width: int, intermediate: int, experts: int, top: int, router: str = "router", expert: str = "e{}",
+                 pieces=("gate", "up", "down")):
+        if not 1 <= top <= experts:
+            raise ValueError(f"a token uses {top} of {experts} experts")
+        self.width, self.intermediate, self.experts, self.top = width, intermediate, experts, top
+        self.router_name, self.expert_name, self.pieces = router, expert, tuple(pieces)
+        self._parts = {}
+        self.router = None        # float32 [experts, W]
+        self.gate_up = None       # [experts, 2F, W]
+        self.down = None          # [experts, W, F]
+
+    def _names(self):
+        gate, up, down = self.pieces
+        for index in range(self.experts):
+            prefix = self.expert_name.format(index)
+            yield index, f"{prefix}.{gate}", f"{prefix}.{up}", f"{prefix}.{down}"
+
+    def param_specs(self):
+        share = self.top / self.experts
+        specs = {self.router_name: ParamSpec((self.experts, self.width), VECTOR, "normal")}
+        for _, gate, up, down in self._names():
+            specs[gate] = ParamSpec((self.intermediate, self.width), share_per_token=share)
+            specs[up] = ParamSpec((self.intermediate, self.width), share_per_token=share)
+            specs[down] = ParamSpec((self.width, self.intermediate), share_per_token=share)
+        return specs
+
+    def assign(self, name, tensor):
+        if name == self.router_name:
+            self.router = tensor
+        else:
+            self._parts[name] = tensor
+
+    def finalize(self):
+        names = list(self._names())
+        self.gate_up = torch.stack([torch.cat([self._parts[gate], self._parts[up]], dim=0) for _, gate, up, _ in names]).contiguous()
+        self.down = torch.stack([self._parts[down] for _, _, _, down in names]).contiguous()
+        self._parts.clear()
+
+    def forward(self, x, ctx):
+        """``x [T, W]`` in the compute type -> float32 ``[T, W]``."""
+        ops = ctx.ops
+        n = x.shape[0]
+        chosen = ctx.empty((n, self.top), dtype=torch.int32)
+        weights = ctx.empty((n, self.top), dtype=torch.float32)
+        ops.route_experts(x, self.router, self.top, chosen, weights)
+        hidden = ctx.empty((n * self.top, self.intermediate))
+        ops.experts_gate_up(x, self.gate_up, chosen, hidden)
+        out = ctx.empty((n, self.width), dtype=torch.float32)
+        ops.experts_down(hidden, self.down, chosen, weights, out)
+        return out

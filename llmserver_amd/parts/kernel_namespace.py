@@ -45,7 +45,61 @@ class KernelNamespace:
         raise NotImplementedError
 
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx, decode_fusion=None):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None):
+        """``sinks [n_q]`` (float32) or None: one more term ``exp(sinks[head])`` in every softmax's denominator, with no
+        key and no value.  ``qkv`` may hold the queries only (``[T, n_q * head_dim]``) where nothing is fused."""
+        raise NotImplementedError
+
+    # A residual stream kept in 32-bit beside activations of the compute type.
+    def embedding_norm(self, table, token_ids, weight, eps, out):
+        """``out [T, W]`` float32 ``= rmsnorm(table[token_ids]) * weight``."""
+        raise NotImplementedError
+
+    def norm_rows(self, x, rows, weight, eps, out):
+        """``out = rmsnorm(x[rows]) * weight`` for a float32 ``x``; ``rows`` int32 or None (all); ``out`` of any type."""
+        raise NotImplementedError
+
+    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out):
+        """``out = x + conv(x)``: a causal convolution over each request's tokens on every channel, ``weight [W, taps]``,
+        tap ``j`` on the token ``taps - 1 - j`` places back; tokens before the step's come from ``state [slots, taps - 1,
+        W]`` (a request's last inputs, oldest first), tokens before the sequence are zeros.  ``x`` float32."""
+        raise NotImplementedError
+
+    def short_conv_keep(self, x, state, state_slots, row_start, row_len, row_ctx):
+        """Move every row's last ``taps - 1`` inputs (the step's, and the state's where the step brings fewer) into ``state``."""
+        raise NotImplementedError
+
+    def scaled_norm_add(self, x, y, weight, scale, eps, out, rounded=None, history=None, before=0, mix=None):
+        """``s = x + rmsnorm(y) * weight * scale`` (``scale`` None: 1), all float32.  Without ``history``: ``out = s``.
+        With ``history [states, T, W]``: ``history[before] = s`` and ``out = sum_{j <= before} mix[j] * history[j]``.
+        ``rounded`` (any type) also gets ``out``."""
+        raise NotImplementedError
+
+    # Attention over a shared low-rank latent.
+    def latent_prepare(self, proj, q_latent, norm_weight, eps, cos_sin, keys, values, table, token_row, positions, page_size,
+                       out_q, n_heads, dim, rot_dim, rank, write_cache=True):
+        """``proj [T, n_heads * (dim + rot_dim) + rank + rot_dim + ...]``: per head ``dim`` plain and ``rot_dim`` rotated
+        query dimensions, then the token's ``rank`` latent dimensions and its ``rot_dim`` shared rotated key dimensions.
+        Writes a cache row ``[rmsnorm(latent) * norm_weight, rotate(key part), zeros]`` of every token as its key and,
+        transposed, as its value, and ``out_q [T, n_heads * D]`` with per head ``[q_latent[h, t], rotate(q's rotated part),
+        zeros]``.  ``cos_sin [T, 2 * pairs]``: neighbouring dimensions (2i, 2i+1) of the first ``2 * pairs`` rotated ones turn."""
+        raise NotImplementedError
+
+    def gate_heads(self, y, proj, gate_column, out):
+        """``out[t, h * v + j] = y[h, t, j] * sigmoid(proj[t, gate_column + h])``."""
+        raise NotImplementedError
+
+    # Routed experts.
+    def route_experts(self, x, router, top, chosen, weights):
+        """Float32 logits ``x router^T``; ``chosen [T, top]`` the largest (first of equals), ``weights`` their softmax."""
+        raise NotImplementedError
+
+    def experts_gate_up(self, x, gate_up, chosen, hidden):
+        """``hidden[t * top + s] = silu(G x_t) * (U x_t)`` with ``[G; U] = gate_up[chosen[t, s]]`` (``[E, 2F, W]``)."""
+        raise NotImplementedError
+
+    def experts_down(self, hidden, down, chosen, weights, out):
+        """``out[t] = sum_s weights[t, s] * down[chosen[t, s]] hidden[t * top + s]``; ``down [E, W, F]``, ``out`` float32."""
         raise NotImplementedError
 
     def sample(self, logits, temperature, uniform, out):

@@ -23,7 +23,10 @@ class Linear(Part):
     """
 
     def __init__(self, in_features: int, pieces: Sequence[str], out_features: Sequence[int], bias: bool = False,
-                 out_float32: bool = False):
+                 out_float32: bool = False, bare_names: bool = False):
+        if bare_names and bias:
+            raise ValueError("a piece whose name is the tensor's has no place for a bias")
+        self.bare_names = bare_names        # the pieces' names are the tensors' names (no ".weight" behind them)
         self.in_features = in_features
         self.pieces = tuple(pieces)
         self.piece_out = tuple(out_features)
@@ -39,12 +42,15 @@ class Linear(Part):
     def param_specs(self):
         specs = {}
         for piece, n in zip(self.pieces, self.piece_out):
-            specs[f"{piece}.weight"] = ParamSpec((n, self.in_features), MATRIX, "normal")
+            specs[piece if self.bare_names else f"{piece}.weight"] = ParamSpec((n, self.in_features), MATRIX, "normal")
             if self.has_bias:
                 specs[f"{piece}.bias"] = ParamSpec((n,), VECTOR, "bias")
         return specs
 
     def assign(self, name, tensor):
+        if self.bare_names:
+            self._w[name] = tensor
+            return
         piece, kind = name.rsplit(".", 1)
         (self._w if kind == "weight" else self._b)[piece] = tensor
 

@@ -11,21 +11,34 @@ from .base import VECTOR, Norm, ParamSpec
 
 
 class RMSNorm(Norm):
-    def __init__(self, width: int, eps: float):
+    """``offset``: what is added to the stored weight before it multiplies (0: the weight as stored; 1: a weight that
+    is stored around zero).  The sum is formed once, in 32-bit, when the tensor has been loaded, so every kernel sees a
+    plain weight.  ``tensor``: the weight's name below the part's own ("" if the part's name is the tensor's)."""
+
+    def __init__(self, width: int, eps: float, offset: float = 0.0, tensor: str = "weight"):
         self.width = width
         self.eps = float(eps)
-        self.weight = None  # float32 [width]
+        self.offset = float(offset)
+        self.tensor = tensor
+        self.weight = None  # float32 [width], the offset added
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.width,), VECTOR, "norm")}
+        return {self.tensor: ParamSpec((self.width,), VECTOR, "bias" if self.offset else "norm")}
 
     def assign(self, name, tensor):
-        assert name == "weight"
-        self.weight = tensor
+        assert name == self.tensor
+        self.weight = tensor + self.offset if self.offset else tensor
 
     def add_norm(self, resid, delta, ctx, rows=None):
         n = resid.shape[0] if rows is None else rows.shape[0]
         out = ctx.empty((n, self.width))
+        if resid.dtype != out.dtype:
+            # A stream that is kept in 32-bit beside 16-bit activations: nothing is added here, rows are normalised
+            # in 32-bit and rounded once for the product that follows.
+            if delta is not None:
+                raise ValueError("a 32-bit residual stream takes its updates where they are made, not in the norm")
+            ctx.ops.norm_rows(resid, rows, self.weight, self.eps, out)
+            return out
         ctx.ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
         return out
 

@@ -39,5 +39,16 @@ class RotaryPosition(PositionEncoding):
         return ctx.computed(("rotary", id(self)), lambda: ctx.ops.rotary_table(ctx.positions, self.rotary_table(ctx.device)))
 
 
+class PairedRotaryPosition(RotaryPosition):
+    """The same angles, for mixers that turn neighbouring dimensions (2i, 2i+1) together instead of (i, i + d/2):
+    ``(u, v) -> (u cos a - v sin a, v cos a + u sin a)`` with ``a = position * theta^(-2i/d)``.  ``rotary_dim`` may be
+    smaller than the vector it is applied to; the dimensions behind it pass unchanged.  The frequencies are formed in
+    64-bit and rounded to 32-bit once; angles, cosines and sines are 32-bit."""
+    pairing = "neighbours"
+
+    def inverse_frequencies(self) -> torch.Tensor:
+        return torch.tensor([self.theta ** (-2.0 * i / self.rotary_dim) for i in range(self.rotary_dim // 2)], dtype=torch.float32)
+
+
 class NoPosition(PositionEncoding):
     """Tokens enter the mixer unrotated."""

@@ -140,7 +140,7 @@ class TorchOps(KernelNamespace):
         values[pages, :, :, slots] = heads[:, n_q + n_kv:].to(values.dtype)
 
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx, decode_fusion=None):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None):
         """Per request row: gather its keys/values through the block table, one softmax over all
         keys a query may see (no tiles, no splits).  ``decode_fusion``: the step's rows bring one token each and
         ``qkv`` is the raw projection, which is left as it is."""
@@ -155,7 +155,7 @@ class TorchOps(KernelNamespace):
             self.qk_norm_rope_kv_write(qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
                                        n_q, n_kv, head_dim, write_cache)
         n = qkv.shape[0]
-        q_all = qkv.view(n, n_q + 2 * n_kv, head_dim)[:, :n_q].float()
+        q_all = qkv.view(n, -1, head_dim)[:, :n_q].float()
         group = n_q // n_kv
         for row in range(table.shape[0]):
             start, length, ctx_len = int(row_start[row]), int(row_len[row]), int(row_ctx[row])
@@ -173,8 +173,124 @@ class TorchOps(KernelNamespace):
             if window:
                 hidden = hidden | (place[None, :] <= q_pos[:, None] - window)
             scores = scores.masked_fill(hidden[None], float("-inf"))
-            result = torch.einsum("hqk,khd->qhd", torch.softmax(scores, dim=-1), v)
+            if sinks is None:
+                weights = torch.softmax(scores, dim=-1)
+            else:
+                top = torch.maximum(scores.max(dim=-1).values, sinks.float()[:, None])
+                weights = torch.exp(scores - top[..., None])
+                weights = weights / (weights.sum(dim=-1) + torch.exp(sinks.float()[:, None] - top))[..., None]
+            result = torch.einsum("hqk,khd->qhd", weights, v)
             out[start:start + length] = result.reshape(length, n_q * head_dim).to(out.dtype)
+
+    # -- a 32-bit residual stream -----------------------------------------------------------------------
+    @staticmethod
+    def _rms(x, eps):
+        return x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+
+    def embedding_norm(self, table, token_ids, weight, eps, out):
+        out.copy_(self._rms(table[token_ids.long()].float(), eps) * weight)
+
+    def norm_rows(self, x, rows, weight, eps, out):
+        picked = x if rows is None else x[rows.long()]
+        out.copy_((self._rms(picked.float(), eps) * weight).to(out.dtype))
+
+    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out):
+        taps = weight.shape[1]
+        result = x.clone()
+        for t in range(x.shape[0]):
+            row, position = int(token_row[t]), int(positions[t])
+            first = position - (t - int(row_start[row]))            # position of the row's first token in this step
+            for j in range(taps):
+                back = taps - 1 - j
+                place = position - back
+                if place < 0:
+                    continue
+                if place >= first:
+                    value = x[t - back]
+                else:
+                    value = state[int(state_slots[row]), taps - 1 - (first - place)]
+                result[t] += weight[:, j] * value
+        out.copy_(result.to(out.dtype))
+
+    def short_conv_keep(self, x, state, state_slots, row_start, row_len, row_ctx):
+        kept = state.shape[1]
+        for row in range(len(row_len)):
+            slot, start, count, end = int(state_slots[row]), int(row_start[row]), int(row_len[row]), int(row_ctx[row])
+            first = end - count
+            old = state[slot].clone()
+            for k in range(kept):
+                place = end - kept + k
+                if place >= first:
+                    state[slot, k] = x[start + place - first]
+                elif place >= 0:
+                    state[slot, k] = old[k + count]
+                else:
+                    state[slot, k] = 0
+
+    def scaled_norm_add(self, x, y, weight, scale, eps, out, rounded=None, history=None, before=0, mix=None):
+        s = x + self._rms(y.float(), eps) * weight * (1.0 if scale is None else scale)
+        if history is not None:
+            history[before] = s
+            s = (history[:before + 1] * mix[:before + 1, None, None]).sum(dim=0)
+        out.copy_(s)
+        if rounded is not None:
+            rounded.copy_(s.to(rounded.dtype))
+
+    # -- attention over a shared latent ------------------------------------------------------------------
+    def latent_prepare(self, proj, q_latent, norm_weight, eps, cos_sin, keys, values, table, token_row, positions, page_size,
+                       out_q, n_heads, dim, rot_dim, rank, write_cache=True):
+        n, width = proj.shape[0], keys.shape[-1]
+        q = proj[:, :n_heads * (dim + rot_dim)].float().view(n, n_heads, dim + rot_dim)
+        down = proj[:, n_heads * (dim + rot_dim):n_heads * (dim + rot_dim) + rank + rot_dim].float()
+        pairs = cos_sin.shape[1] // 2
+        cos, sin = cos_sin[:, :pairs], cos_sin[:, pairs:]
+
+        def turned(x):                                  # x [T, ..., rot_dim]
+            shape = [n] + [1] * (x.dim() - 2) + [pairs]
+            u, v = x[..., 0:2 * pairs:2], x[..., 1:2 * pairs:2]
+            c, s = cos.view(shape), sin.view(shape)
+            return torch.cat([torch.stack([u * c - v * s, v * c + u * s], dim=-1).flatten(-2), x[..., 2 * pairs:]], dim=-1)
+
+        full = torch.zeros((n, n_heads, width), dtype=torch.float32, device=proj.device)
+        full[..., :rank] = q_latent.float().transpose(0, 1)
+        full[..., rank:rank + rot_dim] = turned(q[..., dim:])
+        out_q.copy_(full.view(n, n_heads * width).to(out_q.dtype))
+        if not write_cache:
+            return
+        row = torch.zeros((n, width), dtype=torch.float32, device=proj.device)
+        row[:, :rank] = self._rms(down[:, :rank], eps) * norm_weight
+        row[:, rank:rank + rot_dim] = turned(down[:, rank:])
+        pos = positions.long()
+        pages = table.long()[token_row.long(), pos // page_size]
+        slots = pos % page_size
+        keys[pages, 0, slots, :] = row.to(keys.dtype)
+        values[pages, 0, :, slots] = row.to(values.dtype)
+
+    def gate_heads(self, y, proj, gate_column, out):
+        heads, n, v = y.shape
+        gate = torch.sigmoid(proj[:, gate_column:gate_column + heads].float())
+        out.copy_((y.float().transpose(0, 1) * gate[..., None]).reshape(n, heads * v).to(out.dtype))
+
+    # -- routed experts ----------------------------------------------------------------------------------
+    def route_experts(self, x, router, top, chosen, weights):
+        best = torch.topk(x.float() @ router.float().t(), top, dim=-1)
+        chosen.copy_(best.indices.to(chosen.dtype))
+        weights.copy_(torch.softmax(best.values, dim=-1))
+
+    def experts_gate_up(self, x, gate_up, chosen, hidden):
+        top, inter = chosen.shape[1], hidden.shape[1]
+        for t in range(x.shape[0]):
+            for s in range(top):
+                both = gate_up[int(chosen[t, s])].float() @ x[t].float()
+                gate, up = both[:inter], both[inter:]
+                hidden[t * top + s] = (gate * torch.sigmoid(gate) * up).to(hidden.dtype)
+
+    def experts_down(self, hidden, down, chosen, weights, out):
+        top = chosen.shape[1]
+        out.zero_()
+        for t in range(out.shape[0]):
+            for s in range(top):
+                out[t] += weights[t, s] * (down[int(chosen[t, s])].float() @ hidden[t * top + s].float())
 
     def sample(self, logits, temperature, uniform, out):
         for row in range(logits.shape[0]):
