@@ -48,7 +48,20 @@ struct Geometry {
     int n_q, n_kv, group, gheads, tokens_per_tile, gtiles, page_size, window;
     unsigned page_magic;      // ceil(2^32 / page_size): key / page_size == mulhi(key, page_magic) for key < 2^32 / page_size
     float scale;
+    const float* sinks;       // [n_q] or null: exp(sinks[head]) joins every softmax's denominator (no key, no value)
 };
+
+// What the accumulated output of a pair is multiplied by at the very end: one over the sum of its keys' weights
+// (`total`, taken under the maximum `top`, in natural units with the scale applied) and, where the head has a sink, of
+// the sink's weight too.  The sink enters here and nowhere else, so it counts once however the keys were cut into ranges.
+__device__ __forceinline__ float inverse_of_sum(float total, float top, const float* __restrict__ sinks, int head) {
+    if (sinks == nullptr) return total > 0.f ? 1.f / total : 0.f;
+    if (!(total > 0.f) || top == NEG_INF) return 0.f;
+    const float sink = sinks[head];
+    const float common = fmaxf(top, sink);
+    const float keys = expf(top - common);
+    return keys / (total * keys + expf(sink - common));
+}
 
 // Decode steps (every row brings one token) can leave the per-head norm and the rotation of q and
 // of the new key, and the new key's and value's way into the cache, to this kernel: a wavefront
@@ -573,7 +586,7 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
             weight[w] = m == NEG_INF ? 0.f : expf(m - top);
             total += weight[w] * ranges_sum[first_wave + w][col];
         }
-        const float inv = total > 0.f ? 1.f / total : 0.f;
+        const float inv = inverse_of_sum(total, top, g.sinks, head);
         elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
         for (int c = 0; c < ND; ++c) {
@@ -593,7 +606,7 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     }
     if (!pair_valid) return;
     if (slot < 0) {
-        const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
+        const float inv = inverse_of_sum(run_sum, run_max, g.sinks, head);
         elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
         for (int c = 0; c < ND; ++c) {
@@ -1047,7 +1060,7 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
                 }
                 continue;
             }
-            const float inv = total > 0.f ? 1.f / total : 0.f;
+            const float inv = inverse_of_sum(total, top == NEG_INF ? NEG_INF : top * g.scale, g.sinks, head);
             elem_t* o = out + ((size_t)(row_start[row] + q0 + u * g.tokens_per_tile + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
             for (int c = 0; c < ND; ++c) {
@@ -1079,7 +1092,7 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
             }
             continue;
         }
-        const float inv = total > 0.f ? 1.f / total : 0.f;
+        const float inv = inverse_of_sum(total, run_max[u] == NEG_INF ? NEG_INF : run_max[u] * g.scale, g.sinks, head);
         elem_t* o = out + ((size_t)(row_start[row] + q0 + u * g.tokens_per_tile + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
         for (int c = 0; c < ND; ++c) {
@@ -1265,7 +1278,7 @@ __global__ __launch_bounds__(256) void paged_attention_tile_kernel_f32(
     run_sum += __shfl_xor(run_sum, 16, 64);
     run_sum += __shfl_xor(run_sum, 32, 64);
     if (!pair_valid) return;
-    const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
+    const float inv = inverse_of_sum(run_sum, run_max, g.sinks, head);
     float* o = out + ((size_t)(row_start[row] + q0 + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
     for (int c = 0; c < ND; ++c) *reinterpret_cast<f32x4*>(o + 16 * c) = acc[c] * inv;
@@ -1320,7 +1333,7 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
             weighted += w * sum[i];
         }
         const float total = wave_sum(weighted);
-        if (lane == 0) inv_total = total > 0.f ? 1.f / total : 0.f;
+        if (lane == 0) inv_total = inverse_of_sum(total, top, g.sinks, kv_head * g.group + pair_head_in_group);
     }
     // The partial results do not depend on the weights: their first loads are issued before the barrier.
     const float* acc = part_acc + base * D;
@@ -1392,7 +1405,7 @@ LSA_EXPORT int lsa_paged_attention(
     float scale,
     int window, int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
     int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, int tiles_per_workgroup,
-    int merge_in_workgroup, int tile_halves, hipStream_t stream) {
+    int merge_in_workgroup, int tile_halves, const float* sinks, hipStream_t stream) {
     if (n_items <= 0 && n_tiles <= 0) return 0;
     // decode_fusion (see DecodeFusion::mode): the caller promises that every row of the step brings one token.
     DecodeFusion fusion = {q_weight, k_weight, cos_sin, norm_eps, decode_fusion};
@@ -1400,7 +1413,7 @@ LSA_EXPORT int lsa_paged_attention(
     if (decode_fusion && (!LSA_BF16 || D % 64 != 0 || n_tiles > 0 || (q_weight == nullptr) != (k_weight == nullptr))) return -1;
     Geometry g;
     g.n_q = n_q; g.n_kv = n_kv; g.group = n_q / n_kv; g.gheads = gheads; g.tokens_per_tile = tokens_per_tile;
-    g.gtiles = gtiles; g.page_size = page_size; g.window = window; g.scale = scale;
+    g.gtiles = gtiles; g.page_size = page_size; g.window = window; g.scale = scale; g.sinks = sinks;
     g.page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if (n_tiles > 0) {
 #if LSA_BF16

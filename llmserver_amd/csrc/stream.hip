@@ -1,0 +1,168 @@
+// Row-wise kernels around a residual stream that is kept in float32 whatever the type of the activations:
+// embedding lookup with the norm behind it, a norm of chosen rows, a short causal convolution over time with a
+// per-request state, and the update behind a sublayer (norm of the sublayer's result, per-channel scale, sum, and
+// the weighted sum over the results of the layers so far).  One workgroup per token row; sums of squares, rsqrt and
+// every sum are 32-bit; a result for a 16-bit consumer is rounded once when it is stored.
+#include "common.hpp"
+
+using namespace lsa;
+
+template <typename T>
+__device__ inline float row_square_sum(const T* __restrict__ row, int width, float* scratch) {
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = (float)row[i];
+        sq += v * v;
+    }
+    return block_sum(sq, scratch);
+}
+
+// out[t] = table[ids[t]] * rsqrt(mean(.^2) + eps) * weight.  An id outside the table gives a zero row (the host
+// refuses such ids before the launch).
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_norm_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                                             const float* __restrict__ weight, float eps, float* __restrict__ out,
+                                                             int width, int vocab) {
+    __shared__ float scratch[16];
+    const int id = ids[blockIdx.x];
+    const bool ok = id >= 0 && id < vocab;
+    const T* row = table + (size_t)(ok ? id : 0) * width;
+    const float sq = row_square_sum(row, width, scratch);
+    const float inv = ok ? rsqrtf(sq / (float)width + eps) : 0.f;
+    float* o = out + (size_t)blockIdx.x * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = (float)row[i] * inv * weight[i];
+}
+
+// out[i] = x[rows[i]] * rsqrt(mean(.^2) + eps) * weight (rows == nullptr: every row).
+template <typename O>
+__global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                                        const float* __restrict__ weight, float eps, O* __restrict__ out, int width) {
+    __shared__ float scratch[16];
+    const float* row = x + (size_t)(rows ? rows[blockIdx.x] : blockIdx.x) * width;
+    const float inv = rsqrtf(row_square_sum(row, width, scratch) / (float)width + eps);
+    O* o = out + (size_t)blockIdx.x * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = (O)(row[i] * inv * weight[i]);
+}
+
+// out[t] = x[t] + sum_j w[:, j] * h(position - (taps - 1 - j)), where h(p) is the input at position p of the token's
+// request: a row of this step if the step brings position p, the request's state otherwise (state[slot][k] is the
+// input at position first - kept + k, `first` the position of the step's first token of the request, kept = taps - 1),
+// zero before the sequence starts.
+template <typename O>
+__global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ x, const float* __restrict__ w, int taps,
+                                                         const float* __restrict__ state, const int* __restrict__ slots,
+                                                         const int* __restrict__ token_row, const int* __restrict__ positions,
+                                                         const int* __restrict__ row_start, O* __restrict__ out, int width) {
+    const int t = blockIdx.x;
+    const int row = token_row[t], position = positions[t];
+    const int first = position - (t - row_start[row]);
+    const int kept = taps - 1;
+    const float* mine = state ? state + (size_t)slots[row] * kept * width : nullptr;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float acc = x[(size_t)t * width + c];
+        for (int j = 0; j < taps; ++j) {
+            const int back = kept - j, place = position - back;
+            if (place < 0) continue;
+            float v;
+            if (place >= first) v = x[(size_t)(t - back) * width + c];
+            else if (mine) v = mine[(size_t)(kept - (first - place)) * width + c];
+            else v = 0.f;
+            acc += w[(size_t)c * taps + j] * v;
+        }
+        out[(size_t)t * width + c] = (O)acc;
+    }
+}
+
+// After the step: state[slot][k] = input at position end - kept + k, from the step's rows where it brought that
+// position, from the old state where it did not (k + count then indexes it), zero before the sequence.  A thread
+// owns a channel of a row and goes through k upwards, so what it still has to read lies above what it has written.
+__global__ __launch_bounds__(256) void short_conv_keep_kernel(const float* __restrict__ x, float* __restrict__ state,
+                                                              const int* __restrict__ slots, const int* __restrict__ row_start,
+                                                              const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+                                                              int kept, int width) {
+    const int row = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= width) return;
+    const int count = row_len[row], end = row_ctx[row], start = row_start[row];
+    if (count <= 0) return;
+    const int first = end - count;
+    float* mine = state + (size_t)slots[row] * kept * width;
+    for (int k = 0; k < kept; ++k) {
+        const int place = end - kept + k;
+        float v = 0.f;
+        if (place >= first) v = x[(size_t)(start + place - first) * width + c];
+        else if (place >= 0) v = mine[(size_t)(k + count) * width + c];
+        mine[(size_t)k * width + c] = v;
+    }
+}
+
+// s = x + y * rsqrt(mean(y^2) + eps) * weight * scale.  Without history: out = s.  With history [states][T][W]:
+// history[before] = s and out = sum_{j <= before} mix[j] * history[j].  `rounded` (may be null) gets out as well.
+template <typename Y, typename R>
+__global__ __launch_bounds__(256) void scaled_norm_add_kernel(const float* __restrict__ x, const Y* __restrict__ y,
+                                                              const float* __restrict__ weight, const float* __restrict__ scale, float eps,
+                                                              float* __restrict__ out, R* __restrict__ rounded, float* history,
+                                                              size_t state_stride, int before, const float* __restrict__ mix, int width) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * width;
+    const Y* yr = y + base;
+    const float inv = rsqrtf(row_square_sum(yr, width, scratch) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float s = x[base + i] + (float)yr[i] * inv * weight[i] * (scale ? scale[i] : 1.f);
+        if (history) {
+            history[(size_t)before * state_stride + base + i] = s;
+            float total = 0.f;
+            for (int j = 0; j < before; ++j) total += mix[j] * history[(size_t)j * state_stride + base + i];
+            s = total + mix[before] * s;
+        }
+        out[base + i] = s;
+        if (rounded) rounded[base + i] = (R)s;
+    }
+}
+
+LSA_EXPORT int lsa_embedding_norm(int table_code, const void* table, const int* ids, const float* weight, float eps, float* out,
+                                  int n, int width, int vocab, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (table_code) embedding_norm_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)table, ids, weight, eps, out, width, vocab);
+    else embedding_norm_kernel<float><<<n, 256, 0, stream>>>((const float*)table, ids, weight, eps, out, width, vocab);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_norm_rows(const float* x, const int* rows, const float* weight, float eps, void* out, int out_code, int n_out,
+                             int width, hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    if (out_code) norm_rows_kernel<bf16_t><<<n_out, 256, 0, stream>>>(x, rows, weight, eps, (bf16_t*)out, width);
+    else norm_rows_kernel<float><<<n_out, 256, 0, stream>>>(x, rows, weight, eps, (float*)out, width);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_short_conv(const float* x, const float* w, int taps, const float* state, const int* slots, const int* token_row,
+                              const int* positions, const int* row_start, void* out, int out_code, int n, int width, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (taps < 1 || (taps > 1 && (state == nullptr || slots == nullptr))) return -1;
+    if (out_code) short_conv_kernel<bf16_t><<<n, 256, 0, stream>>>(x, w, taps, state, slots, token_row, positions, row_start, (bf16_t*)out, width);
+    else short_conv_kernel<float><<<n, 256, 0, stream>>>(x, w, taps, state, slots, token_row, positions, row_start, (float*)out, width);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_short_conv_keep(const float* x, float* state, const int* slots, const int* row_start, const int* row_len,
+                                   const int* row_ctx, int kept, int rows, int width, hipStream_t stream) {
+    if (rows <= 0 || kept <= 0) return 0;
+    short_conv_keep_kernel<<<dim3(rows, (width + 255) / 256), 256, 0, stream>>>(x, state, slots, row_start, row_len, row_ctx, kept, width);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_scaled_norm_add(const float* x, const void* y, int y_code, const float* weight, const float* scale, float eps,
+                                   float* out, void* rounded, int rounded_code, float* history, long state_stride, int before,
+                                   const float* mix, int n, int width, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (history != nullptr && (mix == nullptr || before < 0)) return -1;
+#define LSA_LAUNCH(Y, R) scaled_norm_add_kernel<Y, R><<<n, 256, 0, stream>>>(x, (const Y*)y, weight, scale, eps, out, (R*)rounded, history, \
+                                                                            (size_t)state_stride, before, mix, width)
+    if (y_code && rounded_code) LSA_LAUNCH(bf16_t, bf16_t);
+    else if (y_code) LSA_LAUNCH(bf16_t, float);
+    else if (rounded_code) LSA_LAUNCH(float, bf16_t);
+    else LSA_LAUNCH(float, float);
+#undef LSA_LAUNCH
+    LSA_LAUNCH_CHECK();
+}

@@ -26,6 +26,9 @@ FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HEAD_DIMS = tuple(range(16, 257, 16))
 BASE_MODULES = ("elementwise", "rope_kv", "sampling", "gemm")
+# Libraries that only some models call (a 32-bit residual stream, attention over a latent, routed experts): loaded, and
+# compiled if need be, when the first such call is made.
+PART_MODULES = ("stream", "latent", "experts")
 
 
 class KernelBuildError(RuntimeError):
@@ -43,13 +46,13 @@ def module_recipe(name: str) -> Tuple[str, List[str]]:
     if name.startswith("attention_"):
         _, kind, dim = name.split("_")
         return "attention.hip", [f"-DLSA_BF16={1 if kind == 'bf16' else 0}", f"-DLSA_ND={int(dim[1:]) // 16}"]
-    if name in BASE_MODULES:
+    if name in BASE_MODULES or name in PART_MODULES:
         return f"{name}.hip", []
     raise KeyError(f"unknown kernel library {name!r}")
 
 
 def all_modules(head_dims: Iterable[int] = (64, 128)) -> List[str]:
-    names = list(BASE_MODULES)
+    names = list(BASE_MODULES) + list(PART_MODULES)
     for dim in head_dims:
         names += [attention_module(True, dim), attention_module(False, dim)]
     return names

@@ -24,7 +24,18 @@ _SIGNATURES = {
     "lsa_sample_static_max_rows": [],
     "lsa_sample_static_error": [c_int],
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, _P, c_int,
-                            c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
+                            c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P, _P],
+    "lsa_embedding_norm": [c_int, _P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
+    "lsa_norm_rows": [_P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
+    "lsa_short_conv": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_short_conv_keep": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_scaled_norm_add": [_P, _P, c_int, _P, _P, c_float, _P, _P, c_int, _P, c_long, c_int, _P, c_int, c_int, _P],
+    "lsa_latent_prepare": [c_int, _P, c_long, _P, _P, c_float, _P, c_int, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int,
+                           c_int, c_int, c_int, c_int, _P],
+    "lsa_gate_heads": [c_int, _P, _P, c_long, c_int, _P, c_int, c_int, c_int, _P],
+    "lsa_route_experts": [c_int, _P, _P, c_int, c_int, _P, _P, c_int, c_int, _P],
+    "lsa_experts_gate_up": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    "lsa_experts_down": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_attention_workgroup_tiles": [],
     "lsa_attention_tile_page_multiple": [],
     "lsa_attention_tile_halves": [],

@@ -80,6 +80,7 @@ class HipOps(KernelNamespace):
         self._sampling = library.load("sampling")
         self._gemm = library.load("gemm")
         self._attention = {}
+        self._parts_libraries = {}
         self.skinny_rows = SKINNY_GEMM_ROWS
         # Whether projections may fold the residual sum and the norm between two few-row products into their
         # epilogues (see linear_into_stream); off, every such sum and norm is a kernel of its own.
@@ -680,7 +681,7 @@ class HipOps(KernelNamespace):
         return dtype == torch.bfloat16 and head_dim % 64 == 0
 
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx, decode_fusion=None):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None):
         """Attention of the step's tokens over their requests' pages.
 
         ``qkv [T, (n_q + 2 n_kv) * d]`` holds the normalised, rotated queries in its first
@@ -690,9 +691,17 @@ class HipOps(KernelNamespace):
         :meth:`qk_norm_rope_kv_write` before this one: ``qkv`` is then the raw projection, every row of the step
         must bring exactly one token, and the kernel normalises and rotates q and the new key itself and (with
         ``write_cache``) takes the new key and value from ``qkv`` and puts them into the pages.
+
+        Without ``decode_fusion``, ``qkv`` may hold the queries alone (``[T, n_q * d]``).  ``sinks [n_q]`` float32: one
+        more term ``exp(sinks[head])`` in the denominator of every softmax of that head (no key, no value).
         """
         n = qkv.shape[0]
-        _check(qkv, "qkv", None, (n, (n_q + 2 * n_kv) * head_dim))
+        if decode_fusion is None and qkv.shape[1] == n_q * head_dim:
+            _check(qkv, "q", None, (n, n_q * head_dim))
+        else:
+            _check(qkv, "qkv", None, (n, (n_q + 2 * n_kv) * head_dim))
+        if sinks is not None:
+            _check(sinks, "sinks", torch.float32, (n_q,))
         _check(out, "out", qkv.dtype, (n, n_q * head_dim))
         _check(keys, "keys", qkv.dtype)
         _check(values, "values", qkv.dtype)
@@ -760,8 +769,166 @@ class HipOps(KernelNamespace):
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),
             n_merges, n_slots, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), _ptr(tile_slots), n_tiles, float(scale), int(window) if window else 0,
             page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, fusion_mode, _ptr(q_weight), _ptr(k_weight), float(norm_eps),
-            _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), merge_in_workgroup, int(plan.get("tile_halves", 1)), _stream()),
-            "paged_attention")
+            _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), merge_in_workgroup, int(plan.get("tile_halves", 1)), _ptr(sinks),
+            _stream()), "paged_attention")
+
+    # -- a residual stream in float32, attention over a latent, routed experts ---------------------------
+    # (libraries of their own, loaded at the first call: models that have none of these parts never build them)
+    def _part_library(self, name):
+        loaded = self._parts_libraries.get(name)
+        if loaded is None:
+            loaded = self._parts_libraries[name] = library.load(name)
+        return loaded
+
+    def embedding_norm(self, table, token_ids, weight, eps, out):
+        n, width = out.shape
+        _check(table, "table")
+        _check(token_ids, "token_ids", torch.int32, (n,))
+        _check(weight, "weight", torch.float32, (width,))
+        _check(out, "out", torch.float32)
+        if table.shape[1] != width:
+            raise ValueError(f"embedding: table width {table.shape[1]} != out width {width}")
+        _launched(self._part_library("stream").lsa_embedding_norm(_code(table), _ptr(table), _ptr(token_ids), _ptr(weight), float(eps),
+                                                                  _ptr(out), n, width, table.shape[0], _stream()), "embedding_norm")
+
+    def norm_rows(self, x, rows, weight, eps, out):
+        n_out, width = out.shape
+        _check(x, "x", torch.float32)
+        _check(weight, "weight", torch.float32, (width,))
+        _check(out, "out")
+        if x.shape[1] != width:
+            raise ValueError(f"norm_rows: x has width {x.shape[1]}, out {width}")
+        if rows is not None:
+            _check(rows, "rows", torch.int32, (n_out,))
+        elif x.shape[0] != n_out:
+            raise ValueError(f"norm_rows: {x.shape[0]} rows in, {n_out} out")
+        _launched(self._part_library("stream").lsa_norm_rows(_ptr(x), _ptr(rows), _ptr(weight), float(eps), _ptr(out), _code(out), n_out,
+                                                             width, _stream()), "norm_rows")
+
+    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out):
+        n, width = x.shape
+        taps = weight.shape[1]
+        _check(x, "x", torch.float32)
+        _check(weight, "weight", torch.float32, (width, taps))
+        _check(out, "out", None, (n, width))
+        _check(token_row, "token_row", torch.int32, (n,))
+        _check(positions, "positions", torch.int32, (n,))
+        _check(row_start, "row_start", torch.int32)
+        if taps > 1:
+            if state is None or state_slots is None:
+                raise ValueError("a convolution of several taps needs the requests' state and their slots")
+            _check(state, "state", torch.float32, (state.shape[0], taps - 1, width))
+            _check(state_slots, "state_slots", torch.int32, (row_start.shape[0],))
+        _launched(self._part_library("stream").lsa_short_conv(
+            _ptr(x), _ptr(weight), taps, _ptr(state) if taps > 1 else None, _ptr(state_slots) if taps > 1 else None, _ptr(token_row),
+            _ptr(positions), _ptr(row_start), _ptr(out), _code(out), n, width, _stream()), "short_conv")
+
+    def short_conv_keep(self, x, state, state_slots, row_start, row_len, row_ctx):
+        n, width = x.shape
+        rows = row_len.shape[0]
+        _check(x, "x", torch.float32)
+        _check(state, "state", torch.float32, (state.shape[0], state.shape[1], width))
+        for name, tensor in (("state_slots", state_slots), ("row_start", row_start), ("row_len", row_len), ("row_ctx", row_ctx)):
+            _check(tensor, name, torch.int32, (rows,))
+        _launched(self._part_library("stream").lsa_short_conv_keep(_ptr(x), _ptr(state), _ptr(state_slots), _ptr(row_start), _ptr(row_len),
+                                                                   _ptr(row_ctx), state.shape[1], rows, width, _stream()), "short_conv_keep")
+
+    def scaled_norm_add(self, x, y, weight, scale, eps, out, rounded=None, history=None, before=0, mix=None):
+        n, width = x.shape
+        _check(x, "x", torch.float32)
+        _check(y, "y", None, (n, width))
+        _check(weight, "weight", torch.float32, (width,))
+        if scale is not None:
+            _check(scale, "scale", torch.float32, (width,))
+        _check(out, "out", torch.float32, (n, width))
+        if rounded is not None:
+            _check(rounded, "rounded", None, (n, width))
+        if history is not None:
+            _check(history, "history", torch.float32, (history.shape[0], n, width))
+            _check(mix, "mix", torch.float32)
+            if not 0 <= before < history.shape[0] or mix.shape[0] < before + 1:
+                raise ValueError(f"the result would be state {before} of {history.shape[0]}, mixed with {mix.shape[0]} weights")
+            if out.data_ptr() == x.data_ptr():
+                raise ValueError("with a history the result must not overwrite x")
+        _launched(self._part_library("stream").lsa_scaled_norm_add(
+            _ptr(x), _ptr(y), _code(y), _ptr(weight), _ptr(scale), float(eps), _ptr(out), _ptr(rounded),
+            _code(rounded) if rounded is not None else 0, _ptr(history), n * width, int(before), _ptr(mix), n, width, _stream()),
+            "scaled_norm_add")
+
+    def latent_prepare(self, proj, q_latent, norm_weight, eps, cos_sin, keys, values, table, token_row, positions, page_size,
+                       out_q, n_heads, dim, rot_dim, rank, write_cache=True):
+        n = proj.shape[0]
+        _check(proj, "proj")
+        if proj.shape[1] < n_heads * (dim + rot_dim) + rank + rot_dim:
+            raise ValueError(f"proj has {proj.shape[1]} columns, queries and the latent need {n_heads * (dim + rot_dim) + rank + rot_dim}")
+        _check(q_latent, "q_latent", proj.dtype, (n_heads, n, rank))
+        _check(norm_weight, "norm_weight", torch.float32, (rank,))
+        pairs = cos_sin.shape[1] // 2
+        _check(cos_sin, "cos_sin", torch.float32, (n, 2 * pairs))
+        if 2 * pairs > rot_dim:
+            raise ValueError(f"{2 * pairs} dimensions turn, the rotated part has {rot_dim}")
+        pages, row_width = keys.shape[0], keys.shape[-1]
+        _check(keys, "keys", proj.dtype, (pages, 1, page_size, row_width))
+        _check(values, "values", proj.dtype, (pages, 1, row_width, page_size))
+        if rank + rot_dim > row_width:
+            raise ValueError(f"a cache row of {row_width} cannot hold {rank} + {rot_dim} numbers")
+        _check(table, "table", torch.int32)
+        _check(token_row, "token_row", torch.int32, (n,))
+        _check(positions, "positions", torch.int32, (n,))
+        _check(out_q, "out_q", proj.dtype, (n, n_heads * row_width))
+        _launched(self._part_library("latent").lsa_latent_prepare(
+            _code(proj), _ptr(proj), proj.shape[1], _ptr(q_latent), _ptr(norm_weight), float(eps), _ptr(cos_sin), pairs, _ptr(keys),
+            _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions), page_size, _ptr(out_q), n_heads, dim, rot_dim,
+            rank, row_width, 1 if write_cache else 0, n, _stream()), "latent_prepare")
+
+    def gate_heads(self, y, proj, gate_column, out):
+        heads, n, v = y.shape
+        _check(y, "y", out.dtype)
+        _check(proj, "proj", out.dtype)
+        _check(out, "out", None, (n, heads * v))
+        if proj.shape[0] != n or gate_column + heads > proj.shape[1]:
+            raise ValueError(f"gates of {heads} heads from column {gate_column} do not lie in proj {tuple(proj.shape)}")
+        _launched(self._part_library("latent").lsa_gate_heads(_code(out), _ptr(y), _ptr(proj), proj.shape[1], int(gate_column), _ptr(out),
+                                                              heads, v, n, _stream()), "gate_heads")
+
+    def route_experts(self, x, router, top, chosen, weights):
+        n, width = x.shape
+        experts = router.shape[0]
+        _check(x, "x")
+        _check(router, "router", torch.float32, (experts, width))
+        _check(chosen, "chosen", torch.int32, (n, top))
+        _check(weights, "weights", torch.float32, (n, top))
+        if not 1 <= top <= experts or experts > 8192:
+            raise ValueError(f"the router kernel chooses 1 to {min(experts, 8192)} of up to 8192 experts, asked for {top} of {experts}")
+        _launched(self._part_library("experts").lsa_route_experts(_code(x), _ptr(x), _ptr(router), experts, top, _ptr(chosen), _ptr(weights),
+                                                                  n, width, _stream()), "route_experts")
+
+    EXPERT_LDS_BYTES = 64000      # a token's row (gate/up) or its hidden rows (down) lie in LDS
+
+    def experts_gate_up(self, x, gate_up, chosen, hidden):
+        n, width = x.shape
+        experts, top, inter = gate_up.shape[0], chosen.shape[1], hidden.shape[1]
+        _check(x, "x")
+        _check(gate_up, "gate_up", x.dtype, (experts, 2 * inter, width))
+        _check(chosen, "chosen", torch.int32, (n, top))
+        _check(hidden, "hidden", x.dtype, (n * top, inter))
+        if width * x.element_size() > self.EXPERT_LDS_BYTES:
+            raise ValueError(f"the experts' kernels keep a token's row in LDS: width {width} is too large")
+        _launched(self._part_library("experts").lsa_experts_gate_up(_code(x), _ptr(x), _ptr(gate_up), _ptr(chosen), _ptr(hidden), n, top,
+                                                                    inter, width, experts, _stream()), "experts_gate_up")
+
+    def experts_down(self, hidden, down, chosen, weights, out):
+        n, width = out.shape
+        experts, top, inter = down.shape[0], chosen.shape[1], hidden.shape[1]
+        _check(hidden, "hidden", None, (n * top, inter))
+        _check(down, "down", hidden.dtype, (experts, width, inter))
+        _check(chosen, "chosen", torch.int32, (n, top))
+        _check(weights, "weights", torch.float32, (n, top))
+        _check(out, "out", torch.float32)
+        if top * inter * hidden.element_size() > self.EXPERT_LDS_BYTES:
+            raise ValueError(f"the experts' kernels keep a token's {top} hidden rows of {inter} in LDS: too large")
+        _launched(self._part_library("experts").lsa_experts_down(_code(hidden), _ptr(hidden), _ptr(down), _ptr(chosen), _ptr(weights),
+                                                                 _ptr(out), n, top, inter, width, experts, _stream()), "experts_down")
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape

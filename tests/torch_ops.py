@@ -268,7 +268,7 @@ class TorchOps(KernelNamespace):
 
     def gate_heads(self, y, proj, gate_column, out):
         heads, n, v = y.shape
-        gate = torch.sigmoid(proj[:, gate_column:gate_column + heads].float())
+        gate = torch.sigmoid(proj[:, gate_column:gate_column + heads].float()) if gate_column >= 0 else torch.ones(n, heads, device=y.device)
         out.copy_((y.float().transpose(0, 1) * gate[..., None]).reshape(n, heads * v).to(out.dtype))
 
     # -- routed experts ----------------------------------------------------------------------------------
