@@ -14,7 +14,7 @@ template <typename T>
 __device__ inline float wave_dot(const T* __restrict__ w, const T* x_lds, int n, int lane) {
     constexpr int V = Elem<T>::kVec;
     float acc = 0.f;
-    if (n % V == 0 && (reinterpret_cast<size_t>(w) & 15) == 0) {
+    if (n % V == 0 && ((reinterpret_cast<size_t>(w) | reinterpret_cast<size_t>(x_lds)) & 15) == 0) {
         for (int i = lane * V; i < n; i += 64 * V) {
             const Vec16<T> a = load_vec16(w + i);
             const Vec16<T> b = *reinterpret_cast<const Vec16<T>*>(x_lds + i);
@@ -32,7 +32,7 @@ template <typename T>
 __device__ inline void wave_dot2(const T* __restrict__ w0, const T* __restrict__ w1, const T* x_lds, int n, int lane, float& r0, float& r1) {
     constexpr int V = Elem<T>::kVec;
     float a0 = 0.f, a1 = 0.f;
-    if (n % V == 0 && ((reinterpret_cast<size_t>(w0) | reinterpret_cast<size_t>(w1)) & 15) == 0) {
+    if (n % V == 0 && ((reinterpret_cast<size_t>(w0) | reinterpret_cast<size_t>(w1) | reinterpret_cast<size_t>(x_lds)) & 15) == 0) {
         for (int i = lane * V; i < n; i += 64 * V) {
             const Vec16<T> p = load_vec16(w0 + i);
             const Vec16<T> q = load_vec16(w1 + i);
@@ -105,13 +105,17 @@ __global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ x, con
 template <typename T>
 __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ gate_up,
                                                               const int* __restrict__ chosen, T* __restrict__ hidden, int top,
-                                                              int inter, int width, int experts, int columns_per_block) {
+                                                              int inter, int width, int experts, int columns_per_block, bool in_lds) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
-    T* x_lds = reinterpret_cast<T*>(lds_bytes);
     const int pair = blockIdx.x, t = pair / top;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) x_lds[i] = x[(size_t)t * width + i];
-    __syncthreads();
+    const T* x_lds = x + (size_t)t * width;                  // (a row too long for LDS is read where it lies)
+    if (in_lds) {
+        T* staged = reinterpret_cast<T*>(lds_bytes);
+        for (int i = threadIdx.x; i < width; i += blockDim.x) staged[i] = x_lds[i];
+        __syncthreads();
+        x_lds = staged;
+    }
     int expert = chosen[pair];
     expert = expert < 0 ? 0 : expert >= experts ? experts - 1 : expert;
     const T* base = gate_up + (size_t)expert * 2 * inter * width;
@@ -128,13 +132,17 @@ template <typename T>
 __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__ hidden, const T* __restrict__ down,
                                                            const int* __restrict__ chosen, const float* __restrict__ weights,
                                                            float* __restrict__ out, int top, int inter, int width, int experts,
-                                                           int columns_per_block) {
+                                                           int columns_per_block, bool in_lds) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
-    T* h_lds = reinterpret_cast<T*>(lds_bytes);
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
-    for (int i = threadIdx.x; i < top * inter; i += blockDim.x) h_lds[i] = hidden[(size_t)t * top * inter + i];
-    __syncthreads();
+    const T* h_lds = hidden + (size_t)t * top * inter;
+    if (in_lds) {
+        T* staged = reinterpret_cast<T*>(lds_bytes);
+        for (int i = threadIdx.x; i < top * inter; i += blockDim.x) staged[i] = h_lds[i];
+        __syncthreads();
+        h_lds = staged;
+    }
     const int c0 = blockIdx.y * columns_per_block, c1 = min(width, c0 + columns_per_block);
     for (int c = c0 + wave; c < c1; c += waves) {
         float acc = 0.f;
@@ -161,23 +169,25 @@ LSA_EXPORT int lsa_route_experts(int code, const void* x, const float* router, i
 LSA_EXPORT int lsa_experts_gate_up(int code, const void* x, const void* gate_up, const int* chosen, void* hidden, int n, int top,
                                    int inter, int width, int experts, hipStream_t stream) {
     if (n <= 0) return 0;
-    const size_t lds = (size_t)width * (code ? 2 : 4);
-    if (lds > 64000) return -1;
+    size_t lds = (size_t)width * (code ? 2 : 4);
+    const bool in_lds = lds <= 64000;
+    if (!in_lds) lds = 0;
     const int columns = 16;
     dim3 grid(n * top, (inter + columns - 1) / columns);
-    if (code) experts_gate_up_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, chosen, (bf16_t*)hidden, top, inter, width, experts, columns);
-    else experts_gate_up_kernel<float><<<grid, 256, lds, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)hidden, top, inter, width, experts, columns);
+    if (code) experts_gate_up_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, chosen, (bf16_t*)hidden, top, inter, width, experts, columns, in_lds);
+    else experts_gate_up_kernel<float><<<grid, 256, lds, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)hidden, top, inter, width, experts, columns, in_lds);
     LSA_LAUNCH_CHECK();
 }
 
 LSA_EXPORT int lsa_experts_down(int code, const void* hidden, const void* down, const int* chosen, const float* weights, float* out,
                                 int n, int top, int inter, int width, int experts, hipStream_t stream) {
     if (n <= 0) return 0;
-    const size_t lds = (size_t)top * inter * (code ? 2 : 4);
-    if (lds > 64000) return -1;
+    size_t lds = (size_t)top * inter * (code ? 2 : 4);
+    const bool in_lds = lds <= 64000;
+    if (!in_lds) lds = 0;
     const int columns = 16;
     dim3 grid(n, (width + columns - 1) / columns);
-    if (code) experts_down_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)hidden, (const bf16_t*)down, chosen, weights, out, top, inter, width, experts, columns);
-    else experts_down_kernel<float><<<grid, 256, lds, stream>>>((const float*)hidden, (const float*)down, chosen, weights, out, top, inter, width, experts, columns);
+    if (code) experts_down_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)hidden, (const bf16_t*)down, chosen, weights, out, top, inter, width, experts, columns, in_lds);
+    else experts_down_kernel<float><<<grid, 256, lds, stream>>>((const float*)hidden, (const float*)down, chosen, weights, out, top, inter, width, experts, columns, in_lds);
     LSA_LAUNCH_CHECK();
 }

@@ -903,8 +903,6 @@ class HipOps(KernelNamespace):
         _launched(self._part_library("experts").lsa_route_experts(_code(x), _ptr(x), _ptr(router), experts, top, _ptr(chosen), _ptr(weights),
                                                                   n, width, _stream()), "route_experts")
 
-    EXPERT_LDS_BYTES = 64000      # a token's row (gate/up) or its hidden rows (down) lie in LDS
-
     def experts_gate_up(self, x, gate_up, chosen, hidden):
         n, width = x.shape
         experts, top, inter = gate_up.shape[0], chosen.shape[1], hidden.shape[1]
@@ -912,8 +910,6 @@ class HipOps(KernelNamespace):
         _check(gate_up, "gate_up", x.dtype, (experts, 2 * inter, width))
         _check(chosen, "chosen", torch.int32, (n, top))
         _check(hidden, "hidden", x.dtype, (n * top, inter))
-        if width * x.element_size() > self.EXPERT_LDS_BYTES:
-            raise ValueError(f"the experts' kernels keep a token's row in LDS: width {width} is too large")
         _launched(self._part_library("experts").lsa_experts_gate_up(_code(x), _ptr(x), _ptr(gate_up), _ptr(chosen), _ptr(hidden), n, top,
                                                                     inter, width, experts, _stream()), "experts_gate_up")
 
@@ -925,8 +921,6 @@ class HipOps(KernelNamespace):
         _check(chosen, "chosen", torch.int32, (n, top))
         _check(weights, "weights", torch.float32, (n, top))
         _check(out, "out", torch.float32)
-        if top * inter * hidden.element_size() > self.EXPERT_LDS_BYTES:
-            raise ValueError(f"the experts' kernels keep a token's {top} hidden rows of {inter} in LDS: too large")
         _launched(self._part_library("experts").lsa_experts_down(_code(hidden), _ptr(hidden), _ptr(down), _ptr(chosen), _ptr(weights),
                                                                  _ptr(out), n, top, inter, width, experts, _stream()), "experts_down")
 

@@ -179,3 +179,12 @@ def head_scale(config):
     """The design's usual score scale, 1 / sqrt(dimensions of a head's key), for configurations made by tests."""
     sizes = config["layers"][0]["mixer"]
     return 1.0 / math.sqrt(sizes["dim"] + sizes["rot_dim"])
+
+
+def greedy_generate(config, tensors, prompt, count):
+    """``count`` tokens, each the first largest logit behind everything before it (the whole sequence again every time)."""
+    tokens, made = list(prompt), []
+    for _ in range(count):
+        made.append(int(torch.argmax(forward(config, tensors, tokens)[-1])))
+        tokens.append(made[-1])
+    return made
