@@ -131,6 +131,9 @@ class CacheManager:
                 self.layer_in_group[cache] = position
             self.groups.append(group)
         self.num_state_slots = num_state_slots if self.state_specs else 0
+        # One more slot of storage behind the requests': rows of nobody's, which fill a captured step up to its shape,
+        # read and write it (all of them the same one: nobody reads what they leave).
+        self.scratch_state_slot = self.num_state_slots
         self.free_state_slots = list(range(self.num_state_slots - 1, -1, -1))
         self.state: Dict[int, torch.Tensor] = {}
         self.requests: Dict[object, RequestCache] = {}
@@ -146,7 +149,7 @@ class CacheManager:
             group.keys = torch.zeros((n, pages, spec.n_kv_heads, self.page_size, spec.head_dim), device=self.device, dtype=self.dtype)
             group.values = torch.zeros((n, pages, spec.n_kv_heads, spec.head_dim, self.page_size), device=self.device, dtype=self.dtype)
         for cache, spec in self.state_specs.items():
-            self.state[cache] = torch.zeros((max(1, self.num_state_slots), *spec.shape), device=self.device,
+            self.state[cache] = torch.zeros((self.num_state_slots + 1, *spec.shape), device=self.device,
                                             dtype=getattr(torch, spec.dtype))
 
     @staticmethod

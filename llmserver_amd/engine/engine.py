@@ -127,6 +127,10 @@ class Engine:
                                      model_identity=str(getattr(model, "name", "model")))
         self.enable_prefix_caching = config.enable_prefix_caching and self.kv_cache.prefix_caching_possible
         self.runner = ModelRunner(model, self.kv_cache, ops)
+        if self.kv_cache.state_specs:
+            # A step that was started ahead and is then dropped has been through the requests' state already; pages
+            # forgive that (the same values are written again), a state does not.
+            self.launch_ahead = False
         self.sampler = Sampler(self.runner.ops, self.device)
         self._requests_added = 0
         self._text: Dict[str, ByteLevelText] = {}

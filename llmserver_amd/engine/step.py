@@ -85,7 +85,8 @@ class ModelRunner:
         self._flip = 0
         self.vocab = model.head.out_features
         self._mixers = list({id(block.mixer): block.mixer for block in model.blocks}.values())
-        graph_safe = all(mixer.graph_safe for mixer in self._mixers) and not cache.state_specs
+        # (rows of nobody's, which fill a captured step up, keep their state in a slot behind the requests')
+        graph_safe = all(mixer.graph_safe for mixer in self._mixers)
         if use_graphs is None:
             use_graphs = self.device.type == "cuda" and ops.name == "hip"
         self.use_graphs = bool(use_graphs and graph_safe)
@@ -184,7 +185,8 @@ class ModelRunner:
         request_ids = request_ids + [None] * extra_rows
         slots = None
         if self.cache.state_specs:
-            slots = np.asarray([self.cache.record(rid).state_slot for rid in request_ids], dtype=np.int32)
+            slots = np.asarray([self.cache.record(rid).state_slot if rid is not None else self.cache.scratch_state_slot
+                                for rid in request_ids], dtype=np.int32)
         if staging is None:
             self._flip ^= 1
             staging = self._staging[self._flip]

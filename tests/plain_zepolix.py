@@ -25,6 +25,16 @@ import torch
 from safetensors import safe_open
 
 
+def exact(x):
+    return x
+
+
+def rounding_to(dtype):
+    """``x -> x`` rounded to ``dtype`` and widened back: stands where kernels of that type round their results.  With
+    it the same equations say how far a faultless run in that type lies from the exact result on given tokens."""
+    return lambda x: x.to(dtype).to(x.dtype)
+
+
 def read_folder(folder, dtype=torch.float64):
     """config.json as a dict and every tensor of model.safetensors (floats widened to ``dtype``)."""
     with open(os.path.join(folder, "config.json")) as handle:
@@ -91,27 +101,28 @@ def causal_mask(n_tokens):
     return index[None, :] > index[:, None]
 
 
-def latent_attention(h, tensors, prefix, sizes, eps, angle_dtype=torch.float32):
-    """The mixer.  ``sizes``: the layer's ``mixer`` entry of config.json."""
+def latent_attention(h, tensors, prefix, sizes, eps, angle_dtype=torch.float32, r=exact):
+    """The mixer.  ``sizes``: the layer's ``mixer`` entry of config.json.  ``r`` rounds what 16-bit kernels would round:
+    the projections' results, the normed latent, rotated parts, keys and values, the heads' outputs."""
     n = h.shape[0]
     heads, dim, rot_dim, vdim, rank = sizes["heads"], sizes["dim"], sizes["rot_dim"], sizes["vdim"], sizes["kv_rank"]
     positions = torch.arange(n)
-    q = (h @ tensors[prefix + "q"].T).view(n, heads, dim + rot_dim)
+    q = r(h @ tensors[prefix + "q"].T).view(n, heads, dim + rot_dim)
     q_plain, q_rot = q[..., :dim], q[..., dim:]
-    down = h @ tensors[prefix + "dkv"].T
-    latent = norm_plain_weight(down[:, :rank], tensors[prefix + "dkv.norm"], eps)
+    down = r(h @ tensors[prefix + "dkv"].T)
+    latent = r(norm_plain_weight(down[:, :rank], tensors[prefix + "dkv.norm"], eps))
     k_rot = down[:, rank:]                                                          # one for all heads, not normed
-    k_plain = (latent @ tensors[prefix + "uk"].T).view(n, heads, dim)
-    values = (latent @ tensors[prefix + "uv"].T).view(n, heads, vdim)
+    k_plain = r(latent @ tensors[prefix + "uk"].T).view(n, heads, dim)
+    values = r(latent @ tensors[prefix + "uv"].T).view(n, heads, vdim)
     rot = sizes["rot"]
-    q_rot = rotate_pairs(q_rot, positions, rot["base"], rot["dims"], angle_dtype)
-    k_rot = rotate_pairs(k_rot, positions, rot["base"], rot["dims"], angle_dtype)
+    q_rot = r(rotate_pairs(q_rot, positions, rot["base"], rot["dims"], angle_dtype))
+    k_rot = r(rotate_pairs(k_rot, positions, rot["base"], rot["dims"], angle_dtype))
     scores = (torch.einsum("qhd,khd->hqk", q_plain, k_plain) + torch.einsum("qhd,kd->hqk", q_rot, k_rot)) * sizes["scale"]
     scores = scores.masked_fill(causal_mask(n)[None], float("-inf"))
     weights = softmax_with_sink(scores, tensors[prefix + "sink"][:, None])
-    mixed = torch.einsum("hqk,khd->qhd", weights, values)
-    gate = torch.sigmoid(h @ tensors[prefix + "g"].T)                               # [T, heads]
-    return (mixed * gate[..., None]).reshape(n, heads * vdim) @ tensors[prefix + "o"].T
+    mixed = r(torch.einsum("hqk,khd->qhd", r(weights), values))
+    gate = torch.sigmoid(r(h @ tensors[prefix + "g"].T))                            # [T, heads]
+    return r(r(mixed * gate[..., None]).reshape(n, heads * vdim) @ tensors[prefix + "o"].T)
 
 
 def route(h, router_weight, top):
@@ -121,18 +132,18 @@ def route(h, router_weight, top):
     return chosen.indices, torch.softmax(chosen.values, dim=-1)
 
 
-def expert(h, tensors, prefix):
-    gate = h @ tensors[prefix + "gate"].T
-    return ((gate * torch.sigmoid(gate)) * (h @ tensors[prefix + "up"].T)) @ tensors[prefix + "down"].T
+def expert(h, tensors, prefix, r=exact):
+    gate, up = r(h @ tensors[prefix + "gate"].T), r(h @ tensors[prefix + "up"].T)
+    return r(r((gate * torch.sigmoid(gate)) * up) @ tensors[prefix + "down"].T)
 
 
-def routed_experts(h, tensors, prefix, sizes):
+def routed_experts(h, tensors, prefix, sizes, r=exact):
     """Every token's weighted sum of its chosen experts' outputs."""
     indices, weights = route(h, tensors[prefix + "router"], sizes["router"]["top"])
     out = torch.zeros_like(h)
     for token in range(h.shape[0]):
         for index, weight in zip(indices[token].tolist(), weights[token]):
-            out[token] += weight * expert(h[token:token + 1], tensors, f"{prefix}e{index}.")[0]
+            out[token] += weight * expert(h[token:token + 1], tensors, f"{prefix}e{index}.", r)[0]
     return out
 
 
@@ -141,8 +152,9 @@ def depth_average(states, weights):
     return sum(weight * state for weight, state in zip(weights, states))
 
 
-def layer(x, tensors, index, entry, config, angle_dtype=torch.float32):
-    """One layer's result (before the average over depth)."""
+def layer(x, tensors, index, entry, config, angle_dtype=torch.float32, r=exact):
+    """One layer's result (before the average over depth).  The stream itself is never rounded; what the sublayers
+    read of it is (``r``)."""
     eps = config["norm"]["eps"]
     prefix = f"l{index}."
     h = x
@@ -150,28 +162,28 @@ def layer(x, tensors, index, entry, config, angle_dtype=torch.float32):
         h = h + short_convolution(h, tensors[prefix + "canon1"])
     if entry["type"] != "latent_attention":
         raise ValueError(f"no mixer {entry['type']!r} in this design")
-    mixed = latent_attention(h, tensors, prefix + "mix.", entry["mixer"], eps, angle_dtype)
+    mixed = latent_attention(r(h), tensors, prefix + "mix.", entry["mixer"], eps, angle_dtype, r)
     x = x + norm_around_zero(mixed, tensors[prefix + "norm1"], eps) * tensors[prefix + "ls1"]
     if entry.get("mlp") is not None:
         if entry["mlp"]["kind"] != "moe":
             raise ValueError(f"no feed-forward {entry['mlp']['kind']!r} in this design")
-        fed = routed_experts(x, tensors, prefix + "mlp.", entry["mlp"])
+        fed = routed_experts(r(x), tensors, prefix + "mlp.", entry["mlp"], r)
         x = x + norm_around_zero(fed, tensors[prefix + "norm2"], eps) * tensors[prefix + "ls2"]
     return x
 
 
-def forward(config, tensors, tokens, angle_dtype=torch.float32, streams=False):
+def forward(config, tensors, tokens, angle_dtype=torch.float32, streams=False, r=exact):
     """Logits ``[T, vocab]`` of one sequence; with ``streams`` also every layer's result ``[layers, T, W]``."""
     eps = config["norm"]["eps"]
     ids = torch.as_tensor(tokens, dtype=torch.long)
     x = norm_around_zero(tensors["embed"][ids], tensors["embed.norm"], eps)
     states, results = [x], []
     for index, entry in enumerate(config["layers"]):
-        result = layer(x, tensors, index, entry, config, angle_dtype)
+        result = layer(x, tensors, index, entry, config, angle_dtype, r)
         results.append(result)
         states.append(result)
         x = depth_average(states, tensors[f"l{index}.dwa"])
-    logits = norm_around_zero(x, tensors["final.norm"], eps) @ tensors["head"].T
+    logits = r(norm_around_zero(x, tensors["final.norm"], eps)) @ tensors["head"].T
     return (logits, torch.stack(results)) if streams else logits
 
 
