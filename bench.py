@@ -53,13 +53,13 @@ def prefill_flops(model, tokens):
 
 def random_model(name, layers, dtype, seed=0):
     from llmserver_amd.config import config_from_dict, named_size
+    from llmserver_amd.config.named_sizes import with_layers
     from llmserver_amd.kernels import default_ops
-    from llmserver_amd.weights import RandomInit, random_model_on_device
-    raw = named_size(name)
-    full = raw["num_hidden_layers"]
-    raw["num_hidden_layers"] = min(full, layers) if layers else full
-    config = config_from_dict(raw)
-    default_ops().preload([config.head_dim], dtype)
+    from llmserver_amd.parts.base import paged_part
+    from llmserver_amd.weights import RandomInit, build_model, random_model_on_device
+    full = config_from_dict(named_size(name)).num_hidden_layers
+    config = config_from_dict(with_layers(named_size(name), layers))
+    default_ops().preload(sorted({spec.head_dim for spec in map(paged_part, build_model(config).cache_specs().values()) if spec}), dtype)
     log(f"[bench] {name}: drawing random weights")
     model = random_model_on_device(config, "cuda:0", dtype, RandomInit(seed=seed, std=0.02))
     model.name = f"{name}-random"
@@ -75,7 +75,11 @@ def decode_through_engine(model, page_size, batch, context, steps, warmup, seed=
     from llmserver_amd.engine import Engine, RequestStatus
     prompt_tokens = context - steps - warmup
     pages = batch * (-(-(context + 8) // page_size)) + 16
-    engine = Engine(model, None, max_new_tokens=steps + warmup + 8, max_batch_size=batch, max_num_batched_tokens=max(4096, batch * page_size),
+    from llmserver_amd.parts.base import state_part
+    # (a model whose layers carry a state from step to step shares no prompt pages: its prompts go through one common step)
+    shares_pages = not any(state_part(spec) is not None for spec in model.cache_specs().values())
+    budget = max(4096, batch * page_size) if shares_pages else max(4096, batch * prompt_tokens)
+    engine = Engine(model, None, max_new_tokens=steps + warmup + 8, max_batch_size=batch, max_num_batched_tokens=budget,
                     kv_cache_num_blocks=pages, kv_cache_block_size=page_size, stream_text=False, max_completed_requests=0,
                     ignore_eos=True, enable_prefix_caching=True)
     generator = torch.Generator().manual_seed(seed)
@@ -83,7 +87,7 @@ def decode_through_engine(model, page_size, batch, context, steps, warmup, seed=
     prompts = [torch.randint(0, vocab, (prompt_tokens,), generator=generator).tolist() for _ in range(batch)]
     # Every prompt goes through the engine once on its own, which leaves its complete pages in the cache; the requests
     # that are timed then find them, compute the last few tokens of their prompts in one common step, and decode in step.
-    for prompt in prompts:
+    for prompt in prompts if shares_pages else ():
         engine.add_request(None, prompt_token_ids=prompt, max_new_tokens=1)
         while engine.step():
             pass
@@ -193,7 +197,12 @@ def main() -> int:
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points")
     parser.add_argument("--no-extra-points", action="store_true", help="skip the Qwen3-1.7B-sized mixed workload and the Qwen3-32B-sized batch")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--design", default="", choices=("", "zepolix"),
+                        help="instead of the default workload: prefill and decode of this design at a few named sizes, each beside "
+                             "the dense decoder of equal width, depth and active feed-forward size")
     args = parser.parse_args()
+    if args.design:
+        return compare_design(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
@@ -275,6 +284,47 @@ def main() -> int:
     if points:
         result["points"] = points
     print(json.dumps(result), flush=True)
+    return 0
+
+
+DESIGN_SIZES = {"zepolix": (("zepolix-2k", "dense-2k"), ("zepolix-4k", "dense-4k"))}
+
+
+def compare_design(args) -> int:
+    """Prefill (one prompt, arrival to first token) and decode (batch 1, 8, 32 behind 2,048 tokens) of every named size of the
+    design and of the dense decoder beside it, through the same ``Engine.step()``; one JSON line."""
+    import torch
+
+    from llmserver_amd.engine.loading import parse_dtype
+    dtype = parse_dtype(args.dtype)
+    short = "bf16" if dtype == torch.bfloat16 else "fp32"
+    context, steps, warmup = 2048, min(args.steps, 32), min(args.warmup, 4)
+    sizes = {}
+    for pair in DESIGN_SIZES[args.design]:
+        for name in pair:
+            model, config, _ = random_model(name, args.layers, dtype)
+            entry = {"layers": config.num_hidden_layers, "weights_gb_one_row": round(decode_step_bytes(model, 1, 0) / 1e9, 3)}
+            for tokens in (512, args.prefill_tokens):
+                log(f"[bench] {name}: prefill of {tokens} tokens")
+                seconds = prefill_through_engine(model, args.page_size, tokens)
+                entry[f"prefill_{tokens}_ms"] = round(1000.0 * seconds, 3)
+                entry[f"prefill_{tokens}_tok_s"] = round(tokens / seconds, 1)
+                entry[f"prefill_{tokens}_mfma_frac"] = round(prefill_flops(model, tokens) / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)
+            for batch in (1, 8, 32):
+                log(f"[bench] {name}: decode batch {batch} behind {context} tokens")
+                rate, ms, gbs = decode_point(model, args.page_size, batch, context, steps, warmup)
+                entry[f"decode_b{batch}_tok_s"] = round(rate, 1)
+                entry[f"decode_b{batch}_ms_per_step"] = round(ms, 4)
+                entry[f"decode_b{batch}_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
+            sizes[name] = entry
+            del model
+            torch.cuda.empty_cache()
+    first = DESIGN_SIZES[args.design][0][0]
+    print(json.dumps({"metric": f"{args.design} beside the dense decoder: prefill and decode at named sizes (random weights)",
+                      "value": sizes[first]["decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+                      "ms_per_step": sizes[first]["decode_b8_ms_per_step"], "higher_is_better": True, "dtype": short, "data": "synthetic",
+                      "config": {"model": first, "global_batch": 8, "seq_len": context, "timed_through": "Engine.step"}, "sizes": sizes}),
+          flush=True)
     return 0
 
 

@@ -31,6 +31,30 @@ NAMED_SIZES = {
 }
 
 
+
+
+def _zepolix(width, layers, heads, dim, rot_dim, vdim, kv_rank, ff, experts, top, vocab=32768, taps=4):
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": (dim + rot_dim) ** -0.5,
+             "rot": {"base": 10000.0, "dims": rot_dim}}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    return {"architecture": "Zepolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "canon": {"taps": taps},
+            "layers": [{"type": "latent_attention", "mixer": dict(mixer), "mlp": dict(mlp)} for _ in range(layers)]}
+
+
+# Zepolix at sizes that resemble a published mixture-of-experts model's layers (16 heads of 128 + 64 query dimensions and a
+# value size of 128 over a width of 2,048, 64 experts of 1,408 of which a token uses 6; the latent is 192 wide, so that a
+# cache row fills the widest head the attention kernels take), and one twice as wide; and, for each, the dense decoder of
+# this package with the same width, depth, heads and head size whose feed-forward is as large as the experts a token uses.
+NAMED_SIZES.update({
+    "zepolix-2k": _zepolix(2048, 8, 16, 128, 64, 128, 192, 1408, 64, 6),
+    "zepolix-4k": _zepolix(4096, 8, 32, 128, 64, 128, 192, 2048, 32, 4),
+    "dense-2k": dict(model_type="qwen3", num_hidden_layers=8, hidden_size=2048, num_attention_heads=16, num_key_value_heads=8,
+                     head_dim=128, intermediate_size=6 * 1408, vocab_size=32768, rope_theta=10000.0, rms_norm_eps=1e-6),
+    "dense-4k": dict(model_type="qwen3", num_hidden_layers=8, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                     head_dim=128, intermediate_size=4 * 2048, vocab_size=32768, rope_theta=10000.0, rms_norm_eps=1e-6),
+})
+
+
 def named_size(name: str) -> dict:
     """The entry's keys, a copy the caller may change (fewer layers, say)."""
     try:
@@ -41,7 +65,15 @@ def named_size(name: str) -> dict:
 
 def named_config(name: str, layers: Optional[int] = None) -> ModelConfig:
     """The typed configuration of a named size, with at most ``layers`` layers if given (shapes do not depend on depth)."""
-    raw = named_size(name)
+    return config_from_dict(with_layers(named_size(name), layers))
+
+
+def with_layers(raw: dict, layers: Optional[int]) -> dict:
+    """The same configuration with at most ``layers`` layers (0 or None: all), however the architecture counts them."""
+    raw = dict(raw)
     if layers:
-        raw["num_hidden_layers"] = min(int(raw["num_hidden_layers"]), int(layers))
-    return config_from_dict(raw)
+        if isinstance(raw.get("layers"), list):
+            raw["layers"] = raw["layers"][:int(layers)]
+        else:
+            raw["num_hidden_layers"] = min(int(raw["num_hidden_layers"]), int(layers))
+    return raw

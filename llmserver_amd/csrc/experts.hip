@@ -53,26 +53,18 @@ __device__ inline void wave_dot2(const T* __restrict__ w0, const T* __restrict__
     r1 = wave_sum(a1);
 }
 
-// One workgroup per token: logits of all experts (a wavefront per expert in turn), then wavefront 0 picks the `top`
-// largest (the lowest index among equal ones) and writes their softmax.  Dynamic LDS: a float per expert.
-template <typename T>
-__global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ x, const float* __restrict__ router, int experts, int top,
-                                                    int* __restrict__ chosen, float* __restrict__ weights, int width) {
+// One wavefront per token: the `top` largest of the token's float32 logits (the lowest index among equal ones) and
+// their softmax.  The logits themselves are a float32 matrix product made before this kernel.  A lane keeps the logits
+// of experts lane, lane + 64, ... in LDS (its own entries only: nothing crosses lanes through LDS), and every lane ends
+// each round with the same (best, where).
+__global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict__ all_logits, int experts, int top,
+                                                        int* __restrict__ chosen, float* __restrict__ weights, int n_tokens) {
     extern __shared__ float lds[];
-    float* logits = lds;
-    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
-    const T* row = x + (size_t)t * width;
-    for (int e = wave; e < experts; e += waves) {
-        const float* r = router + (size_t)e * width;
-        float acc = 0.f;
-        for (int i = lane; i < width; i += 64) acc += r[i] * (float)row[i];
-        acc = wave_sum(acc);
-        if (lane == 0) logits[e] = acc;
-    }
-    __syncthreads();
-    if (wave) return;
-    // Every lane ends each round with the same (best, where), so nothing crosses lanes through LDS: the lane that
-    // owns an entry of `logits` (entry % 64) is the only one that reads it and the one that strikes it out.
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (t >= n_tokens) return;
+    float* logits = lds + (size_t)wave * experts;
+    for (int e = lane; e < experts; e += 64) logits[e] = all_logits[(size_t)t * experts + e];
     float largest = 0.f, total = 0.f;
     for (int k = 0; k < top; ++k) {
         float best = NEG_INF;
@@ -128,12 +120,15 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
 }
 
 // grid (tokens, blocks of output columns): out[t][c] = sum_s weights[t][s] * (D_s[c] . hidden[t * top + s]).
+// A wavefront owns a column: every lane adds up its share of all `top` dot products, weighted, and the lanes' sums meet
+// once at the end; the loads of all pairs' rows are independent of one another.
 template <typename T>
 __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__ hidden, const T* __restrict__ down,
                                                            const int* __restrict__ chosen, const float* __restrict__ weights,
                                                            float* __restrict__ out, int top, int inter, int width, int experts,
                                                            int columns_per_block, bool in_lds) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
+    constexpr int V = Elem<T>::kVec;
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const T* h_lds = hidden + (size_t)t * top * inter;
@@ -143,26 +138,45 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
         __syncthreads();
         h_lds = staged;
     }
+    const bool vectors = inter % V == 0 && ((reinterpret_cast<size_t>(down) | reinterpret_cast<size_t>(h_lds)) & 15) == 0;
     const int c0 = blockIdx.y * columns_per_block, c1 = min(width, c0 + columns_per_block);
     for (int c = c0 + wave; c < c1; c += waves) {
         float acc = 0.f;
-        for (int s = 0; s < top; ++s) {
-            int expert = chosen[(size_t)t * top + s];
-            expert = expert < 0 ? 0 : expert >= experts ? experts - 1 : expert;
-            const T* row = down + ((size_t)expert * width + c) * inter;
-            acc += weights[(size_t)t * top + s] * wave_dot(row, h_lds + (size_t)s * inter, inter, lane);
+        if (vectors) {
+            // The pairs' rows end to end are one long vector of top * inter / V pieces, spread over the lanes: every
+            // lane is busy whatever the experts' size, and its loads do not wait for one another.
+            const int pieces = inter / V, all = top * pieces;
+            for (int p = lane; p < all; p += 64) {
+                const int s = p / pieces, i = (p - s * pieces) * V;
+                int expert = chosen[(size_t)t * top + s];
+                expert = expert < 0 ? 0 : expert >= experts ? experts - 1 : expert;
+                const Vec16<T> a = load_vec16(down + ((size_t)expert * width + c) * inter + i);
+                const Vec16<T> b = *reinterpret_cast<const Vec16<T>*>(h_lds + (size_t)s * inter + i);
+                float part = 0.f;
+#pragma unroll
+                for (int k = 0; k < V; ++k) part += (float)a.v[k] * (float)b.v[k];
+                acc += weights[(size_t)t * top + s] * part;
+            }
+        } else {
+            for (int s = 0; s < top; ++s) {
+                int expert = chosen[(size_t)t * top + s];
+                expert = expert < 0 ? 0 : expert >= experts ? experts - 1 : expert;
+                const T* row = down + ((size_t)expert * width + c) * inter;
+                const T* h = h_lds + (size_t)s * inter;
+                float part = 0.f;
+                for (int i = lane; i < inter; i += 64) part += (float)row[i] * (float)h[i];
+                acc += weights[(size_t)t * top + s] * part;
+            }
         }
+        acc = wave_sum(acc);
         if (lane == 0) out[(size_t)t * width + c] = acc;
     }
 }
 
-LSA_EXPORT int lsa_route_experts(int code, const void* x, const float* router, int experts, int top, int* chosen, float* weights,
-                                 int n, int width, hipStream_t stream) {
+LSA_EXPORT int lsa_route_top(const float* logits, int experts, int top, int* chosen, float* weights, int n, hipStream_t stream) {
     if (n <= 0) return 0;
-    if (top < 1 || top > experts || (size_t)experts * 4 > 60000) return -1;
-    const size_t lds = (size_t)experts * sizeof(float);
-    if (code) route_kernel<bf16_t><<<n, 256, lds, stream>>>((const bf16_t*)x, router, experts, top, chosen, weights, width);
-    else route_kernel<float><<<n, 256, lds, stream>>>((const float*)x, router, experts, top, chosen, weights, width);
+    if (top < 1 || top > experts || (size_t)experts * 16 > 60000) return -1;
+    route_top_kernel<<<(n + 3) / 4, 256, (size_t)experts * 4 * sizeof(float), stream>>>(logits, experts, top, chosen, weights, n);
     LSA_LAUNCH_CHECK();
 }
 
@@ -185,9 +199,179 @@ LSA_EXPORT int lsa_experts_down(int code, const void* hidden, const void* down, 
     size_t lds = (size_t)top * inter * (code ? 2 : 4);
     const bool in_lds = lds <= 64000;
     if (!in_lds) lds = 0;
-    const int columns = 16;
+    const int columns = 4;
     dim3 grid(n, (width + columns - 1) / columns);
     if (code) experts_down_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)hidden, (const bf16_t*)down, chosen, weights, out, top, inter, width, experts, columns, in_lds);
     else experts_down_kernel<float><<<grid, 256, lds, stream>>>((const float*)hidden, (const float*)down, chosen, weights, out, top, inter, width, experts, columns, in_lds);
+    LSA_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Many tokens (portions of prompts, large batches): the pairs are sorted by expert, each expert's pairs padded to whole
+// tiles of TILE_M rows, and one MFMA product per tile multiplies the tile's rows with its expert's matrix, so an expert's
+// weights are read once per tile of 64 pairs instead of once per pair.  bfloat16 only (the float32 path keeps the
+// kernels above).
+//
+// sort: one workgroup.  sorted[i] = pair at padded place i (-1: padding), tile_expert[j] = expert of tile j (-1: no tile).
+// The order of an expert's pairs among themselves is whatever the atomics give; every pair's row is computed on its
+// own, so the results do not depend on it.
+constexpr int TILE_M = 64;
+
+__global__ __launch_bounds__(1024) void experts_sort_kernel(const int* __restrict__ chosen, int n_pairs, int experts,
+                                                            int* __restrict__ sorted, int* __restrict__ tile_expert, int max_tiles) {
+    extern __shared__ int lds_ints[];
+    int* counts = lds_ints;
+    int* offsets = lds_ints + experts;
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
+    for (int i = threadIdx.x; i < max_tiles * TILE_M; i += blockDim.x) sorted[i] = -1;
+    for (int j = threadIdx.x; j < max_tiles; j += blockDim.x) tile_expert[j] = -1;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = chosen[p];
+        if (e >= 0 && e < experts) atomicAdd(&counts[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int running = 0;
+        for (int e = 0; e < experts; ++e) {
+            offsets[e] = running;
+            const int tiles = (counts[e] + TILE_M - 1) / TILE_M;
+            for (int j = 0; j < tiles; ++j) tile_expert[running / TILE_M + j] = e;
+            running += tiles * TILE_M;
+            counts[e] = 0;                       // from here on: how many of the expert's pairs have a place
+        }
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = chosen[p];
+        if (e >= 0 && e < experts) sorted[offsets[e] + atomicAdd(&counts[e], 1)] = p;
+    }
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// C = A . B^T for one tile of 64 sorted pairs and 128 rows of the expert's matrix (K contiguous in both).
+//   GATED: B's 128 rows are 64 gate rows f0 .. f0 + 63 and their 64 up rows; the result is silu(gate) * up, 64 columns.
+//   Rows of A: a[(sorted[i] / pair_div)] (pair_div = top for the tokens' rows, 1 for the pairs' hidden rows).
+// Four wavefronts, each 32 rows x 64 columns (GATED: 32 gate columns and their 32 up columns): 2 x 4 MFMA tiles of
+// 16 x 16, k in steps of 32.  A slab of BK columns of K of both operands goes through LDS (rows padded by 16 bytes).
+template <int BK, bool GATED, typename O>
+__global__ __launch_bounds__(256) void experts_tile_kernel(const bf16_t* __restrict__ a, int a_stride, int pair_div,
+                                                           const bf16_t* __restrict__ b, long expert_stride, int b_rows, int b_up_offset,
+                                                           const int* __restrict__ sorted, const int* __restrict__ tile_expert,
+                                                           O* __restrict__ out, int out_stride, int n_out, int k) {
+    constexpr int ROW = BK + 8;                                    // elements of a padded row in LDS
+    __shared__ __align__(16) bf16_t a_lds[TILE_M * ROW];
+    __shared__ __align__(16) bf16_t b_lds[128 * ROW];
+    __shared__ int rows_of[TILE_M];
+    const int expert = tile_expert[blockIdx.x];
+    if (expert < 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, quad = lane >> 4;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    if (threadIdx.x < TILE_M) rows_of[threadIdx.x] = sorted[blockIdx.x * TILE_M + threadIdx.x];
+    __syncthreads();
+    const int n0 = blockIdx.y * (GATED ? 64 : 128);                // first output column of the block
+    const bf16_t* bm = b + (size_t)expert * expert_stride;
+    // which rows of B the block's 128 LDS rows are: GATED: LDS row r < 64 -> gate row n0 + r, r >= 64 -> up row n0 + r - 64
+    auto b_row = [&](int r) {
+        int row = GATED ? (r < 64 ? n0 + r : b_up_offset + n0 + r - 64) : n0 + r;
+        const int last = GATED ? (r < 64 ? n_out - 1 : b_up_offset + n_out - 1) : n_out - 1;
+        return row > last ? last : row;                            // (columns beyond the matrix repeat its last row; never stored)
+    };
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int PIECES = BK / 8;                                 // 16-byte pieces of a row of a slab
+    for (int k0 = 0; k0 < k; k0 += BK) {
+        for (int i = threadIdx.x; i < TILE_M * PIECES; i += 256) {
+            const int r = i / PIECES, piece = i - r * PIECES;
+            const int pair = rows_of[r];
+            const bf16_t* src = a + (size_t)(pair < 0 ? 0 : pair / pair_div) * a_stride + k0 + 8 * piece;
+            *reinterpret_cast<bf16x8*>(a_lds + r * ROW + 8 * piece) = *reinterpret_cast<const bf16x8*>(src);
+        }
+        for (int i = threadIdx.x; i < 128 * PIECES; i += 256) {
+            const int r = i / PIECES, piece = i - r * PIECES;
+            const bf16_t* src = bm + (size_t)b_row(r) * k + k0 + 8 * piece;
+            *reinterpret_cast<bf16x8*>(b_lds + r * ROW + 8 * piece) = *reinterpret_cast<const bf16x8*>(src);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 32) {
+            bf16x8 av[2], bv[4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) av[i] = *reinterpret_cast<const bf16x8*>(a_lds + (wave_m * 32 + 16 * i + col) * ROW + kk + 8 * quad);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // GATED: tiles 0, 1 are the wavefront's 32 gate columns, tiles 2, 3 their up columns
+                const int r = GATED ? (j < 2 ? wave_n * 32 + 16 * j : 64 + wave_n * 32 + 16 * (j - 2)) : wave_n * 64 + 16 * j;
+                bv[j] = *reinterpret_cast<const bf16x8*>(b_lds + (r + col) * ROW + kk + 8 * quad);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    // lane holds rows 4 * quad + r of each 16 x 16 tile, column col
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int pair = rows_of[wave_m * 32 + 16 * i + 4 * quad + r];
+            if (pair < 0) continue;
+            O* o = out + (size_t)pair * out_stride;
+            if (GATED) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int f = n0 + wave_n * 32 + 16 * j + col;
+                    const float g = acc[i][j][r], u = acc[i][j + 2][r];
+                    if (f < n_out) o[f] = (O)(g / (1.f + expf(-g)) * u);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int c = n0 + wave_n * 64 + 16 * j + col;
+                    if (c < n_out) o[c] = (O)acc[i][j][r];
+                }
+            }
+        }
+}
+
+// out[t][c] = sum_s weights[t][s] * y[t * top + s][c]
+__global__ __launch_bounds__(256) void experts_combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
+                                                              float* __restrict__ out, int top, int width) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < top; ++s) acc += weights[(size_t)t * top + s] * y[((size_t)t * top + s) * width + c];
+        out[(size_t)t * width + c] = acc;
+    }
+}
+
+LSA_EXPORT int lsa_experts_tile_rows() { return TILE_M; }
+
+// Sorted, tiled products for bfloat16: hidden = silu(G x) * (U x) and y = D hidden for all pairs, then the weighted sums.
+// Scratch: sorted [max_tiles * 64] and tile_expert [max_tiles] ints, y [pairs, width] floats; max_tiles >= ceil(pairs / 64) + experts.
+LSA_EXPORT int lsa_experts_tiled(const void* x, const void* gate_up, const void* down, const int* chosen, const float* weights,
+                                 void* hidden, float* y, float* out, int* sorted, int* tile_expert, int max_tiles, int n, int top,
+                                 int inter, int width, int experts, hipStream_t stream) {
+    if (n <= 0) return 0;
+    const int pairs = n * top;
+    if (width % 32 || inter % 32 || max_tiles < (pairs + TILE_M - 1) / TILE_M + experts || (size_t)experts * 8 > 60000) return -1;
+    experts_sort_kernel<<<1, 1024, (size_t)experts * 2 * sizeof(int), stream>>>(chosen, pairs, experts, sorted, tile_expert, max_tiles);
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* gu = (const bf16_t*)gate_up;
+    const bf16_t* dn = (const bf16_t*)down;
+    bf16_t* hb = (bf16_t*)hidden;
+    dim3 grid1(max_tiles, (inter + 63) / 64), grid2(max_tiles, (width + 127) / 128);
+    if (width % 64 == 0) experts_tile_kernel<64, true, bf16_t><<<grid1, 256, 0, stream>>>(xb, width, top, gu, (long)2 * inter * width, 2 * inter, inter, sorted, tile_expert, hb, inter, inter, width);
+    else experts_tile_kernel<32, true, bf16_t><<<grid1, 256, 0, stream>>>(xb, width, top, gu, (long)2 * inter * width, 2 * inter, inter, sorted, tile_expert, hb, inter, inter, width);
+    if (inter % 64 == 0) experts_tile_kernel<64, false, float><<<grid2, 256, 0, stream>>>(hb, inter, 1, dn, (long)width * inter, width, 0, sorted, tile_expert, y, width, width, inter);
+    else experts_tile_kernel<32, false, float><<<grid2, 256, 0, stream>>>(hb, inter, 1, dn, (long)width * inter, width, 0, sorted, tile_expert, y, width, width, inter);
+    experts_combine_kernel<<<n, 256, 0, stream>>>(y, weights, out, top, width);
     LSA_LAUNCH_CHECK();
 }

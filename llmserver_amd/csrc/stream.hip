@@ -48,28 +48,33 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict_
 // request: a row of this step if the step brings position p, the request's state otherwise (state[slot][k] is the
 // input at position first - kept + k, `first` the position of the step's first token of the request, kept = taps - 1),
 // zero before the sequence starts.
-template <typename O>
+template <typename O, int V>
 __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ x, const float* __restrict__ w, int taps,
                                                          const float* __restrict__ state, const int* __restrict__ slots,
                                                          const int* __restrict__ token_row, const int* __restrict__ positions,
                                                          const int* __restrict__ row_start, O* __restrict__ out, int width) {
+    // V (1 or 4) neighbouring channels a thread: the rows it reads are 16-byte pieces where the width allows.
     const int t = blockIdx.x;
     const int row = token_row[t], position = positions[t];
     const int first = position - (t - row_start[row]);
     const int kept = taps - 1;
     const float* mine = state ? state + (size_t)slots[row] * kept * width : nullptr;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) {
-        float acc = x[(size_t)t * width + c];
+    for (int c = threadIdx.x * V; c < width; c += blockDim.x * V) {
+        float acc[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] = x[(size_t)t * width + c + v];
         for (int j = 0; j < taps; ++j) {
             const int back = kept - j, place = position - back;
             if (place < 0) continue;
-            float v;
-            if (place >= first) v = x[(size_t)(t - back) * width + c];
-            else if (mine) v = mine[(size_t)(kept - (first - place)) * width + c];
-            else v = 0.f;
-            acc += w[(size_t)c * taps + j] * v;
+            const float* src;
+            if (place >= first) src = x + (size_t)(t - back) * width + c;
+            else if (mine) src = mine + (size_t)(kept - (first - place)) * width + c;
+            else continue;
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v] += w[(size_t)(c + v) * taps + j] * src[v];
         }
-        out[(size_t)t * width + c] = (O)acc;
+#pragma unroll
+        for (int v = 0; v < V; ++v) out[(size_t)t * width + c + v] = (O)acc[v];
     }
 }
 
@@ -98,25 +103,71 @@ __global__ __launch_bounds__(256) void short_conv_keep_kernel(const float* __res
 
 // s = x + y * rsqrt(mean(y^2) + eps) * weight * scale.  Without history: out = s.  With history [states][T][W]:
 // history[before] = s and out = sum_{j <= before} mix[j] * history[j].  `rounded` (may be null) gets out as well.
-template <typename Y, typename R>
+template <typename Y, typename R, int V>
 __global__ __launch_bounds__(256) void scaled_norm_add_kernel(const float* __restrict__ x, const Y* __restrict__ y,
                                                               const float* __restrict__ weight, const float* __restrict__ scale, float eps,
                                                               float* __restrict__ out, R* __restrict__ rounded, float* history,
                                                               size_t state_stride, int before, const float* __restrict__ mix, int width) {
+    // V (1 or 4) neighbouring elements a thread; the first CACHE pieces of y stay in registers between the two passes.
+    constexpr int CACHE = 4;
     __shared__ float scratch[16];
     const size_t base = (size_t)blockIdx.x * width;
     const Y* yr = y + base;
-    const float inv = rsqrtf(row_square_sum(yr, width, scratch) / (float)width + eps);
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float s = x[base + i] + (float)yr[i] * inv * weight[i] * (scale ? scale[i] : 1.f);
-        if (history) {
-            history[(size_t)before * state_stride + base + i] = s;
-            float total = 0.f;
-            for (int j = 0; j < before; ++j) total += mix[j] * history[(size_t)j * state_stride + base + i];
-            s = total + mix[before] * s;
+    const int stride = blockDim.x * V;
+    float kept[CACHE][V];
+    float sq = 0.f;
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = threadIdx.x * V + k * stride;
+        if (i < width) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                kept[k][v] = (float)yr[i + v];
+                sq += kept[k][v] * kept[k][v];
+            }
         }
-        out[base + i] = s;
-        if (rounded) rounded[base + i] = (R)s;
+    }
+    for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride)
+#pragma unroll
+        for (int v = 0; v < V; ++v) sq += (float)yr[i + v] * (float)yr[i + v];
+    const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
+    auto finish = [&](int i, const float (&yv)[V]) {
+        float s[V], total[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            s[v] = x[base + i + v] + yv[v] * inv * weight[i + v] * (scale ? scale[i + v] : 1.f);
+            total[v] = 0.f;
+        }
+        if (history) {
+            for (int j = 0; j < before; ++j) {
+                const float m = mix[j];
+                const float* h = history + (size_t)j * state_stride + base + i;
+#pragma unroll
+                for (int v = 0; v < V; ++v) total[v] += m * h[v];
+            }
+            const float m = mix[before];
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                history[(size_t)before * state_stride + base + i + v] = s[v];
+                s[v] = total[v] + m * s[v];
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            out[base + i + v] = s[v];
+            if (rounded) rounded[base + i + v] = (R)s[v];
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = threadIdx.x * V + k * stride;
+        if (i < width) finish(i, kept[k]);
+    }
+    for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
+        float yv[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) yv[v] = (float)yr[i + v];
+        finish(i, yv);
     }
 }
 
@@ -140,8 +191,10 @@ LSA_EXPORT int lsa_short_conv(const float* x, const float* w, int taps, const fl
                               const int* positions, const int* row_start, void* out, int out_code, int n, int width, hipStream_t stream) {
     if (n <= 0) return 0;
     if (taps < 1 || (taps > 1 && (state == nullptr || slots == nullptr))) return -1;
-    if (out_code) short_conv_kernel<bf16_t><<<n, 256, 0, stream>>>(x, w, taps, state, slots, token_row, positions, row_start, (bf16_t*)out, width);
-    else short_conv_kernel<float><<<n, 256, 0, stream>>>(x, w, taps, state, slots, token_row, positions, row_start, (float*)out, width);
+#define LSA_LAUNCH(O, V) short_conv_kernel<O, V><<<n, 256, 0, stream>>>(x, w, taps, state, slots, token_row, positions, row_start, (O*)out, width)
+    if (width % 4 == 0) { if (out_code) LSA_LAUNCH(bf16_t, 4); else LSA_LAUNCH(float, 4); }
+    else { if (out_code) LSA_LAUNCH(bf16_t, 1); else LSA_LAUNCH(float, 1); }
+#undef LSA_LAUNCH
     LSA_LAUNCH_CHECK();
 }
 
@@ -157,12 +210,14 @@ LSA_EXPORT int lsa_scaled_norm_add(const float* x, const void* y, int y_code, co
                                    const float* mix, int n, int width, hipStream_t stream) {
     if (n <= 0) return 0;
     if (history != nullptr && (mix == nullptr || before < 0)) return -1;
-#define LSA_LAUNCH(Y, R) scaled_norm_add_kernel<Y, R><<<n, 256, 0, stream>>>(x, (const Y*)y, weight, scale, eps, out, (R*)rounded, history, \
-                                                                            (size_t)state_stride, before, mix, width)
+#define LSA_LAUNCH_V(Y, R, V) scaled_norm_add_kernel<Y, R, V><<<n, 256, 0, stream>>>(x, (const Y*)y, weight, scale, eps, out, (R*)rounded, history, \
+                                                                                  (size_t)state_stride, before, mix, width)
+#define LSA_LAUNCH(Y, R) do { if (width % 4 == 0) LSA_LAUNCH_V(Y, R, 4); else LSA_LAUNCH_V(Y, R, 1); } while (0)
     if (y_code && rounded_code) LSA_LAUNCH(bf16_t, bf16_t);
     else if (y_code) LSA_LAUNCH(bf16_t, float);
     else if (rounded_code) LSA_LAUNCH(float, bf16_t);
     else LSA_LAUNCH(float, float);
 #undef LSA_LAUNCH
+#undef LSA_LAUNCH_V
     LSA_LAUNCH_CHECK();
 }

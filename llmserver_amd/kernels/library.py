@@ -33,8 +33,10 @@ _SIGNATURES = {
     "lsa_latent_prepare": [c_int, _P, c_long, _P, _P, c_float, _P, c_int, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int,
                            c_int, c_int, c_int, c_int, _P],
     "lsa_gate_heads": [c_int, _P, _P, c_long, c_int, _P, c_int, c_int, c_int, _P],
-    "lsa_route_experts": [c_int, _P, _P, c_int, c_int, _P, _P, c_int, c_int, _P],
+    "lsa_route_top": [_P, c_int, c_int, _P, _P, c_int, _P],
     "lsa_experts_gate_up": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    "lsa_experts_tile_rows": [],
+    "lsa_experts_tiled": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_experts_down": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_attention_workgroup_tiles": [],
     "lsa_attention_tile_page_multiple": [],

@@ -892,16 +892,18 @@ class HipOps(KernelNamespace):
                                                               heads, v, n, _stream()), "gate_heads")
 
     def route_experts(self, x, router, top, chosen, weights):
+        """The logits are a float32 product of the library (no reduced-precision mode), the choice and the softmax a kernel."""
         n, width = x.shape
         experts = router.shape[0]
         _check(x, "x")
         _check(router, "router", torch.float32, (experts, width))
         _check(chosen, "chosen", torch.int32, (n, top))
         _check(weights, "weights", torch.float32, (n, top))
-        if not 1 <= top <= experts or experts > 8192:
-            raise ValueError(f"the router kernel chooses 1 to {min(experts, 8192)} of up to 8192 experts, asked for {top} of {experts}")
-        _launched(self._part_library("experts").lsa_route_experts(_code(x), _ptr(x), _ptr(router), experts, top, _ptr(chosen), _ptr(weights),
-                                                                  n, width, _stream()), "route_experts")
+        if not 1 <= top <= experts or experts > 3072:
+            raise ValueError(f"the router kernel chooses 1 to {min(experts, 3072)} of up to 3072 experts, asked for {top} of {experts}")
+        logits = torch.mm(x if x.dtype == torch.float32 else x.float(), router.t())
+        _launched(self._part_library("experts").lsa_route_top(_ptr(logits), experts, top, _ptr(chosen), _ptr(weights), n, _stream()),
+                  "route_top")
 
     def experts_gate_up(self, x, gate_up, chosen, hidden):
         n, width = x.shape
@@ -923,6 +925,30 @@ class HipOps(KernelNamespace):
         _check(out, "out", torch.float32)
         _launched(self._part_library("experts").lsa_experts_down(_code(hidden), _ptr(hidden), _ptr(down), _ptr(chosen), _ptr(weights),
                                                                  _ptr(out), n, top, inter, width, experts, _stream()), "experts_down")
+
+    def experts_sorted(self, x, gate_up, down, chosen, weights, out) -> bool:
+        """Offered in bfloat16 for widths and expert sizes in steps of 32, and taken where the step has more (token,
+        expert) pairs than there are experts: below that every pair streaming its own expert reads no more."""
+        n, width = x.shape
+        experts, top, inter = gate_up.shape[0], chosen.shape[1], down.shape[2]
+        if x.dtype != torch.bfloat16 or width % 32 or inter % 32 or n * top <= experts or experts > 4096:
+            return False
+        _check(x, "x")
+        _check(gate_up, "gate_up", x.dtype, (experts, 2 * inter, width))
+        _check(down, "down", x.dtype, (experts, width, inter))
+        _check(chosen, "chosen", torch.int32, (n, top))
+        _check(weights, "weights", torch.float32, (n, top))
+        _check(out, "out", torch.float32, (n, width))
+        lib = self._part_library("experts")
+        tile = lib.lsa_experts_tile_rows()
+        max_tiles = -(-n * top // tile) + experts
+        hidden = torch.empty((n * top, inter), device=x.device, dtype=x.dtype)
+        y = torch.empty((n * top, width), device=x.device, dtype=torch.float32)
+        scratch = torch.empty((max_tiles * (tile + 1),), device=x.device, dtype=torch.int32)
+        _launched(lib.lsa_experts_tiled(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(hidden), _ptr(y), _ptr(out),
+                                        _ptr(scratch), scratch[max_tiles * tile:].data_ptr(), max_tiles, n, top, inter, width, experts,
+                                        _stream()), "experts_tiled")
+        return True
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape

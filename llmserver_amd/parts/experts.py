@@ -58,8 +58,10 @@ class RoutedExperts(FeedForward):
         chosen = ctx.empty((n, self.top), dtype=torch.int32)
         weights = ctx.empty((n, self.top), dtype=torch.float32)
         ops.route_experts(x, self.router, self.top, chosen, weights)
+        out = ctx.empty((n, self.width), dtype=torch.float32)
+        if ops.experts_sorted(x, self.gate_up, self.down, chosen, weights, out):       # many tokens: pairs sorted by expert
+            return out
         hidden = ctx.empty((n * self.top, self.intermediate))
         ops.experts_gate_up(x, self.gate_up, chosen, hidden)
-        out = ctx.empty((n, self.width), dtype=torch.float32)
         ops.experts_down(hidden, self.down, chosen, weights, out)
         return out

@@ -106,6 +106,12 @@ class KernelNamespace:
         raise NotImplementedError
 
     # -- what a namespace may offer; the answers here mean "not offered" --------------------------------------------
+    def experts_sorted(self, x, gate_up, down, chosen, weights, out) -> bool:
+        """Both products of the routed experts and the weighted sum for all of the step's tokens at once, the (token,
+        expert) pairs sorted by expert so that an expert's matrices are read once per tile of pairs: ``out`` as
+        :meth:`experts_down` leaves it.  False: not done (not offered, or it would not pay for these sizes)."""
+        return False
+
     def check_cache_geometry(self, cache_specs, page_size: int, num_pages=None) -> None:
         """Raise ``ValueError`` for a cache that the kernels cannot read (asked before anything is allocated):
         ``page_size`` keys a page, ``num_pages`` pages (one number, or one per group of caches; None: not said)."""

@@ -173,6 +173,38 @@ def test_routed_experts(ops, dtype, experts, top, width, inter):
     close(results[0][3], results[1][3], dtype, "out")
 
 
+@pytest.mark.parametrize("experts, top, width, inter, tokens", [(5, 2, 64, 32, 40), (12, 3, 96, 160, 333), (70, 6, 256, 96, 200), (3, 1, 32, 64, 700)])
+def test_sorted_expert_products_equal_the_per_pair_ones(ops, experts, top, width, inter, tokens):
+    """Many tokens: the pairs sorted by expert and multiplied tile by tile give what every pair alone gives."""
+    print(f"sorted experts {experts} {top} {width} {inter} {tokens}", flush=True)
+    twin, dtype = TorchOps(), torch.bfloat16
+    x = torch.randn(tokens, width, device="cuda").to(dtype)
+    router = torch.randn(experts, width, device="cuda")
+    if experts > 4:
+        router[3] *= 0.0
+        router[3] -= 100.0 * x.float().mean(dim=0)                 # an expert that (almost) nobody chooses
+    gate_up = (torch.randn(experts, 2 * inter, width, device="cuda") / width ** 0.5).to(dtype)
+    down = (torch.randn(experts, width, inter, device="cuda") / inter ** 0.5).to(dtype)
+    chosen = torch.empty(tokens, top, dtype=torch.int32, device="cuda")
+    weights = torch.empty(tokens, top, device="cuda")
+    ops.route_experts(x, router, top, chosen, weights)
+    out = torch.empty(tokens, width, device="cuda")
+    assert ops.experts_sorted(x, gate_up, down, chosen, weights, out)
+    hidden = torch.empty(tokens * top, inter, device="cuda", dtype=dtype)
+    single = torch.empty(tokens, width, device="cuda")
+    ops.experts_gate_up(x, gate_up, chosen, hidden)
+    ops.experts_down(hidden, down, chosen, weights, single)
+    close(out, single, dtype, "sorted against per pair")
+    some = min(50, tokens)
+    part = slice(0, some)
+    want_hidden = torch.empty(some * top, inter, device="cuda", dtype=dtype)
+    want = torch.empty(some, width, device="cuda")
+    twin.experts_gate_up(x[part], gate_up, chosen[part], want_hidden)
+    twin.experts_down(want_hidden, down, chosen[part], weights[part], want)
+    close(out[part], want, dtype, "sorted against the twin")
+    assert not ops.experts_sorted(x[:1], gate_up, down, chosen[:1], weights[:1], out[:1]) or top > experts
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_a_sink_counts_once_however_the_keys_are_cut(ops, dtype):
     """Attention with a sink over one key-value head against the twin: a prompt whole (workgroups of tiles), single

@@ -12,12 +12,32 @@ import torch
 
 import plain_zepolix as plain
 import traces
-from helpers import check_against_rounded_oracle, random_tokens, relative_error
+from helpers import random_tokens, relative_error
 from tiny_zepolix import CASES, model_folder, plain_logits, plain_model
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 pytestmark = pytest.mark.gpu
 BF16 = plain.rounding_to(torch.bfloat16)
+
+
+def check_rounding(engine_errors, rounded_errors, what, factor=1.25):
+    """A bfloat16 run against what the plain implementation loses when it rounds where 16-bit kernels round, position by
+    position on the same sequences.  Routed experts make the spread heavy-tailed: where two router logits lie a rounding
+    apart, either run may choose the other expert, each at places of its own, and such a place is off by many times the
+    usual error, and so are the places behind it that attend to it: a handful of such events decides the tail of a few
+    thousand places, so the two tails differ by a factor of two between seeds.  The median is therefore held tightly
+    (within ``factor``), the 90th percentile within 1.3 times that, and the tail by its weight: at most 2.5 times as many
+    places far off (ten times the rounded oracle's median) as the rounded oracle has, and two in a hundred."""
+    engine, rounded = np.asarray(engine_errors, dtype=np.float64), np.asarray(rounded_errors, dtype=np.float64)
+    assert np.isfinite(engine).all() and len(engine) >= 48, what
+    middle = float(np.median(rounded))
+    figures = {"median": (np.median(engine), middle, factor), "90th percentile": (np.quantile(engine, 0.9), np.quantile(rounded, 0.9), 1.3 * factor)}
+    far = (float(np.mean(engine > 10 * middle)), float(np.mean(rounded > 10 * middle)))
+    print(f"  {what}: " + ", ".join(f"{name} {ours:.2e} / {theirs:.2e}" for name, (ours, theirs, _) in figures.items()) +
+          f", far off {far[0]:.3f} / {far[1]:.3f}", flush=True)
+    for name, (ours, theirs, allowed) in figures.items():
+        assert ours <= allowed * theirs, f"{what}: {name} error {ours:.3e} is more than {allowed} x the rounded oracle's {theirs:.3e}"
+    assert far[0] <= 2.5 * far[1] + 0.02, f"{what}: {far[0]:.3f} of the places are far off, {far[1]:.3f} of the rounded oracle's"
 
 
 def rounded_logits(case, tokens):
@@ -72,7 +92,7 @@ def test_all_schedules_match_the_plain_implementation(case, dtype, tmp_path):
         for rid, tokens in requests.items():
             exact = plain_logits(case, tuple(tokens)).numpy()
             lost += [relative_error(row, want) for row, want in zip(rounded_logits(case, tuple(tokens)), exact)]
-        check_against_rounded_oracle(errors, lost, f"case {case} against the plain implementation")
+        check_rounding(errors, lost, f"case {case} against the plain implementation")
     # the same request cut differently agrees with itself
     between = []
     for index in range(5):
@@ -84,7 +104,7 @@ def test_all_schedules_match_the_plain_implementation(case, dtype, tmp_path):
                 else:
                     between.append(relative_error(b, a))
     if between:
-        check_against_rounded_oracle(between, lost, f"case {case} between two cuts of the same request", factor=2.0)
+        check_rounding(between, lost, f"case {case} between two cuts of the same request", factor=2.0)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -104,7 +124,7 @@ def test_long_decoding_from_the_first_token(dtype, tmp_path):
             errors.append(relative_error(results[("long", position)], expected[position]))
     if errors:
         lost = [relative_error(row, want) for row, want in zip(rounded_logits(case, tuple(tokens)), expected)]
-        check_against_rounded_oracle(errors, lost, "long decoding")
+        check_rounding(errors, lost, "long decoding")
 
 
 def test_greedy_generation_through_the_entry_point():
