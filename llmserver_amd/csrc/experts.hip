@@ -139,23 +139,31 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
         h_lds = staged;
     }
     const bool vectors = inter % V == 0 && ((reinterpret_cast<size_t>(down) | reinterpret_cast<size_t>(h_lds)) & 15) == 0;
+    // the token's experts and weights, read once (a lookup per piece below would be a trip to memory each)
+    constexpr int MOST = 128;
+    __shared__ int expert_of[MOST];
+    __shared__ float weight_of[MOST];
+    for (int s = threadIdx.x; s < min(top, MOST); s += blockDim.x) {
+        const int expert = chosen[(size_t)t * top + s];
+        expert_of[s] = expert < 0 ? 0 : expert >= experts ? experts - 1 : expert;
+        weight_of[s] = weights[(size_t)t * top + s];
+    }
+    __syncthreads();
     const int c0 = blockIdx.y * columns_per_block, c1 = min(width, c0 + columns_per_block);
     for (int c = c0 + wave; c < c1; c += waves) {
         float acc = 0.f;
-        if (vectors) {
+        if (vectors && top <= MOST) {
             // The pairs' rows end to end are one long vector of top * inter / V pieces, spread over the lanes: every
             // lane is busy whatever the experts' size, and its loads do not wait for one another.
             const int pieces = inter / V, all = top * pieces;
             for (int p = lane; p < all; p += 64) {
                 const int s = p / pieces, i = (p - s * pieces) * V;
-                int expert = chosen[(size_t)t * top + s];
-                expert = expert < 0 ? 0 : expert >= experts ? experts - 1 : expert;
-                const Vec16<T> a = load_vec16(down + ((size_t)expert * width + c) * inter + i);
+                const Vec16<T> a = load_vec16(down + ((size_t)expert_of[s] * width + c) * inter + i);
                 const Vec16<T> b = *reinterpret_cast<const Vec16<T>*>(h_lds + (size_t)s * inter + i);
                 float part = 0.f;
 #pragma unroll
                 for (int k = 0; k < V; ++k) part += (float)a.v[k] * (float)b.v[k];
-                acc += weights[(size_t)t * top + s] * part;
+                acc += weight_of[s] * part;
             }
         } else {
             for (int s = 0; s < top; ++s) {
@@ -196,9 +204,9 @@ LSA_EXPORT int lsa_experts_gate_up(int code, const void* x, const void* gate_up,
 LSA_EXPORT int lsa_experts_down(int code, const void* hidden, const void* down, const int* chosen, const float* weights, float* out,
                                 int n, int top, int inter, int width, int experts, hipStream_t stream) {
     if (n <= 0) return 0;
-    size_t lds = (size_t)top * inter * (code ? 2 : 4);
-    const bool in_lds = lds <= 64000;
-    if (!in_lds) lds = 0;
+    // (a block takes four columns: staging the token's hidden rows in LDS would cost as much as it reads of the weights)
+    const size_t lds = 0;
+    const bool in_lds = false;
     const int columns = 4;
     dim3 grid(n, (width + columns - 1) / columns);
     if (code) experts_down_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)hidden, (const bf16_t*)down, chosen, weights, out, top, inter, width, experts, columns, in_lds);
@@ -254,16 +262,19 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 // C = A . B^T for one tile of 64 sorted pairs and 128 rows of the expert's matrix (K contiguous in both).
 //   GATED: B's 128 rows are 64 gate rows f0 .. f0 + 63 and their 64 up rows; the result is silu(gate) * up, 64 columns.
 //   Rows of A: a[(sorted[i] / pair_div)] (pair_div = top for the tokens' rows, 1 for the pairs' hidden rows).
-// Four wavefronts, each 32 rows x 64 columns (GATED: 32 gate columns and their 32 up columns): 2 x 4 MFMA tiles of
-// 16 x 16, k in steps of 32.  A slab of BK columns of K of both operands goes through LDS (rows padded by 16 bytes).
-template <int BK, bool GATED, typename O>
+// Four wavefronts, each 32 rows x 16 NT columns (GATED: half of them gate columns, half their up columns): 2 x NT MFMA
+// tiles of 16 x 16, k in steps of 32.  A slab of BK columns of K of both operands goes through LDS (rows padded by 16
+// bytes).  NT = 4 where an expert has few pairs (its weights bound the time), 8 where it has many (every operand read
+// from LDS then feeds more products, which is what bounds a tile of 4).
+template <int BK, bool GATED, typename O, int NT>
 __global__ __launch_bounds__(256) void experts_tile_kernel(const bf16_t* __restrict__ a, int a_stride, int pair_div,
                                                            const bf16_t* __restrict__ b, long expert_stride, int b_rows, int b_up_offset,
                                                            const int* __restrict__ sorted, const int* __restrict__ tile_expert,
                                                            O* __restrict__ out, int out_stride, int n_out, int k) {
     constexpr int ROW = BK + 8;                                    // elements of a padded row in LDS
     __shared__ __align__(16) bf16_t a_lds[TILE_M * ROW];
-    __shared__ __align__(16) bf16_t b_lds[128 * ROW];
+    constexpr int BN = 32 * NT;                                    // rows of B a block takes
+    __shared__ __align__(16) bf16_t b_lds[BN * ROW];
     __shared__ int rows_of[TILE_M];
     const int expert = tile_expert[blockIdx.x];
     if (expert < 0) return;
@@ -271,48 +282,72 @@ __global__ __launch_bounds__(256) void experts_tile_kernel(const bf16_t* __restr
     const int wave_m = wave >> 1, wave_n = wave & 1;
     if (threadIdx.x < TILE_M) rows_of[threadIdx.x] = sorted[blockIdx.x * TILE_M + threadIdx.x];
     __syncthreads();
-    const int n0 = blockIdx.y * (GATED ? 64 : 128);                // first output column of the block
+    const int n0 = blockIdx.y * (GATED ? BN / 2 : BN);             // first output column of the block
     const bf16_t* bm = b + (size_t)expert * expert_stride;
-    // which rows of B the block's 128 LDS rows are: GATED: LDS row r < 64 -> gate row n0 + r, r >= 64 -> up row n0 + r - 64
+    // which rows of B the block's LDS rows are: GATED: the first half gate rows n0 + r, the second half their up rows
     auto b_row = [&](int r) {
-        int row = GATED ? (r < 64 ? n0 + r : b_up_offset + n0 + r - 64) : n0 + r;
-        const int last = GATED ? (r < 64 ? n_out - 1 : b_up_offset + n_out - 1) : n_out - 1;
+        int row = GATED ? (r < BN / 2 ? n0 + r : b_up_offset + n0 + r - BN / 2) : n0 + r;
+        const int last = GATED ? (r < BN / 2 ? n_out - 1 : b_up_offset + n_out - 1) : n_out - 1;
         return row > last ? last : row;                            // (columns beyond the matrix repeat its last row; never stored)
     };
-    f32x4 acc[2][4];
+    f32x4 acc[2][NT];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     constexpr int PIECES = BK / 8;                                 // 16-byte pieces of a row of a slab
+    constexpr int A_LOADS = TILE_M * PIECES / 256, B_LOADS = BN * PIECES / 256;      // 16-byte loads of a thread per slab
+    // A thread's pieces of a slab: the same rows and places in every slab, so their addresses are made once.  The next
+    // slab's pieces travel into registers while this slab is multiplied, and go to LDS when everybody is through with it.
+    const bf16_t* a_src[A_LOADS];
+    const bf16_t* b_src[B_LOADS];
+    int a_dst[A_LOADS], b_dst[B_LOADS];
+#pragma unroll
+    for (int u = 0; u < A_LOADS; ++u) {
+        const int i = threadIdx.x + 256 * u, r = i / PIECES, piece = i - r * PIECES;
+        const int pair = rows_of[r];
+        a_src[u] = a + (size_t)(pair < 0 ? 0 : pair / pair_div) * a_stride + 8 * piece;
+        a_dst[u] = r * ROW + 8 * piece;
+    }
+#pragma unroll
+    for (int u = 0; u < B_LOADS; ++u) {
+        const int i = threadIdx.x + 256 * u, r = i / PIECES, piece = i - r * PIECES;
+        b_src[u] = bm + (size_t)b_row(r) * k + 8 * piece;
+        b_dst[u] = r * ROW + 8 * piece;
+    }
+    bf16x8 a_next[A_LOADS], b_next[B_LOADS];
+#pragma unroll
+    for (int u = 0; u < A_LOADS; ++u) a_next[u] = *reinterpret_cast<const bf16x8*>(a_src[u]);
+#pragma unroll
+    for (int u = 0; u < B_LOADS; ++u) b_next[u] = *reinterpret_cast<const bf16x8*>(b_src[u]);
     for (int k0 = 0; k0 < k; k0 += BK) {
-        for (int i = threadIdx.x; i < TILE_M * PIECES; i += 256) {
-            const int r = i / PIECES, piece = i - r * PIECES;
-            const int pair = rows_of[r];
-            const bf16_t* src = a + (size_t)(pair < 0 ? 0 : pair / pair_div) * a_stride + k0 + 8 * piece;
-            *reinterpret_cast<bf16x8*>(a_lds + r * ROW + 8 * piece) = *reinterpret_cast<const bf16x8*>(src);
-        }
-        for (int i = threadIdx.x; i < 128 * PIECES; i += 256) {
-            const int r = i / PIECES, piece = i - r * PIECES;
-            const bf16_t* src = bm + (size_t)b_row(r) * k + k0 + 8 * piece;
-            *reinterpret_cast<bf16x8*>(b_lds + r * ROW + 8 * piece) = *reinterpret_cast<const bf16x8*>(src);
-        }
+#pragma unroll
+        for (int u = 0; u < A_LOADS; ++u) *reinterpret_cast<bf16x8*>(a_lds + a_dst[u]) = a_next[u];
+#pragma unroll
+        for (int u = 0; u < B_LOADS; ++u) *reinterpret_cast<bf16x8*>(b_lds + b_dst[u]) = b_next[u];
         __syncthreads();
+        if (k0 + BK < k) {
+#pragma unroll
+            for (int u = 0; u < A_LOADS; ++u) a_next[u] = *reinterpret_cast<const bf16x8*>(a_src[u] + k0 + BK);
+#pragma unroll
+            for (int u = 0; u < B_LOADS; ++u) b_next[u] = *reinterpret_cast<const bf16x8*>(b_src[u] + k0 + BK);
+        }
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 32) {
-            bf16x8 av[2], bv[4];
+            bf16x8 av[2], bv[NT];
 #pragma unroll
             for (int i = 0; i < 2; ++i) av[i] = *reinterpret_cast<const bf16x8*>(a_lds + (wave_m * 32 + 16 * i + col) * ROW + kk + 8 * quad);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                // GATED: tiles 0, 1 are the wavefront's 32 gate columns, tiles 2, 3 their up columns
-                const int r = GATED ? (j < 2 ? wave_n * 32 + 16 * j : 64 + wave_n * 32 + 16 * (j - 2)) : wave_n * 64 + 16 * j;
+            for (int j = 0; j < NT; ++j) {
+                // GATED: the first half of a wavefront's tiles are its gate columns, the second half their up columns
+                const int r = GATED ? (j < NT / 2 ? wave_n * (BN / 4) + 16 * j : BN / 2 + wave_n * (BN / 4) + 16 * (j - NT / 2))
+                                    : wave_n * (BN / 2) + 16 * j;
                 bv[j] = *reinterpret_cast<const bf16x8*>(b_lds + (r + col) * ROW + kk + 8 * quad);
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     }
@@ -326,15 +361,15 @@ __global__ __launch_bounds__(256) void experts_tile_kernel(const bf16_t* __restr
             O* o = out + (size_t)pair * out_stride;
             if (GATED) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int f = n0 + wave_n * 32 + 16 * j + col;
-                    const float g = acc[i][j][r], u = acc[i][j + 2][r];
+                for (int j = 0; j < NT / 2; ++j) {
+                    const int f = n0 + wave_n * (BN / 4) + 16 * j + col;
+                    const float g = acc[i][j][r], u = acc[i][j + NT / 2][r];
                     if (f < n_out) o[f] = (O)(g / (1.f + expf(-g)) * u);
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int c = n0 + wave_n * 64 + 16 * j + col;
+                for (int j = 0; j < NT; ++j) {
+                    const int c = n0 + wave_n * (BN / 2) + 16 * j + col;
                     if (c < n_out) o[c] = (O)acc[i][j][r];
                 }
             }
@@ -367,11 +402,21 @@ LSA_EXPORT int lsa_experts_tiled(const void* x, const void* gate_up, const void*
     const bf16_t* gu = (const bf16_t*)gate_up;
     const bf16_t* dn = (const bf16_t*)down;
     bf16_t* hb = (bf16_t*)hidden;
-    dim3 grid1(max_tiles, (inter + 63) / 64), grid2(max_tiles, (width + 127) / 128);
-    if (width % 64 == 0) experts_tile_kernel<64, true, bf16_t><<<grid1, 256, 0, stream>>>(xb, width, top, gu, (long)2 * inter * width, 2 * inter, inter, sorted, tile_expert, hb, inter, inter, width);
-    else experts_tile_kernel<32, true, bf16_t><<<grid1, 256, 0, stream>>>(xb, width, top, gu, (long)2 * inter * width, 2 * inter, inter, sorted, tile_expert, hb, inter, inter, width);
-    if (inter % 64 == 0) experts_tile_kernel<64, false, float><<<grid2, 256, 0, stream>>>(hb, inter, 1, dn, (long)width * inter, width, 0, sorted, tile_expert, y, width, width, inter);
-    else experts_tile_kernel<32, false, float><<<grid2, 256, 0, stream>>>(hb, inter, 1, dn, (long)width * inter, width, 0, sorted, tile_expert, y, width, width, inter);
+    const bool many = pairs >= 16 * experts;                    // pairs to an expert: wide tiles pay
+#define LSA_TILES(BK, NT) do { \
+        dim3 grid1(max_tiles, (inter + 16 * NT - 1) / (16 * NT)), grid2(max_tiles, (width + 32 * NT - 1) / (32 * NT)); \
+        if (!second) experts_tile_kernel<BK, true, bf16_t, NT><<<grid1, 256, 0, stream>>>(xb, width, top, gu, (long)2 * inter * width, 2 * inter, inter, sorted, tile_expert, hb, inter, inter, width); \
+        else experts_tile_kernel<BK, false, float, NT><<<grid2, 256, 0, stream>>>(hb, inter, 1, dn, (long)width * inter, width, 0, sorted, tile_expert, y, width, width, inter); \
+    } while (0)
+    for (int pass = 0; pass < 2; ++pass) {
+        const bool second = pass == 1;
+        const bool wide_slab = (second ? inter : width) % 64 == 0;
+        if (wide_slab && many) LSA_TILES(64, 8);
+        else if (wide_slab) LSA_TILES(64, 4);
+        else if (many) LSA_TILES(32, 8);
+        else LSA_TILES(32, 4);
+    }
+#undef LSA_TILES
     experts_combine_kernel<<<n, 256, 0, stream>>>(y, weights, out, top, width);
     LSA_LAUNCH_CHECK();
 }

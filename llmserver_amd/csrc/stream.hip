@@ -50,19 +50,21 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict_
 // zero before the sequence starts.
 template <typename O, int V>
 __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ x, const float* __restrict__ w, int taps,
-                                                         const float* __restrict__ state, const int* __restrict__ slots,
+                                                         float* state, const int* __restrict__ slots,
                                                          const int* __restrict__ token_row, const int* __restrict__ positions,
-                                                         const int* __restrict__ row_start, O* __restrict__ out, int width) {
+                                                         const int* __restrict__ row_start, O* __restrict__ out, int width, int keep) {
     // V (1 or 4) neighbouring channels a thread: the rows it reads are 16-byte pieces where the width allows.
+    // keep (only in steps in which every row brings one token, so that a row's state is one workgroup's): the state
+    // moves on by this token here, in the thread that has just read its channels, instead of in a launch of its own.
     const int t = blockIdx.x;
     const int row = token_row[t], position = positions[t];
     const int first = position - (t - row_start[row]);
     const int kept = taps - 1;
-    const float* mine = state ? state + (size_t)slots[row] * kept * width : nullptr;
+    float* mine = state ? state + (size_t)slots[row] * kept * width : nullptr;
     for (int c = threadIdx.x * V; c < width; c += blockDim.x * V) {
-        float acc[V];
+        float acc[V], own[V];
 #pragma unroll
-        for (int v = 0; v < V; ++v) acc[v] = x[(size_t)t * width + c + v];
+        for (int v = 0; v < V; ++v) acc[v] = own[v] = x[(size_t)t * width + c + v];
         for (int j = 0; j < taps; ++j) {
             const int back = kept - j, place = position - back;
             if (place < 0) continue;
@@ -75,6 +77,13 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict
         }
 #pragma unroll
         for (int v = 0; v < V; ++v) out[(size_t)t * width + c + v] = (O)acc[v];
+        if (keep && mine) {
+            for (int k = 0; k + 1 < kept; ++k)
+#pragma unroll
+                for (int v = 0; v < V; ++v) mine[(size_t)k * width + c + v] = mine[(size_t)(k + 1) * width + c + v];
+#pragma unroll
+            for (int v = 0; v < V; ++v) mine[(size_t)(kept - 1) * width + c + v] = own[v];
+        }
     }
 }
 
@@ -187,11 +196,12 @@ LSA_EXPORT int lsa_norm_rows(const float* x, const int* rows, const float* weigh
     LSA_LAUNCH_CHECK();
 }
 
-LSA_EXPORT int lsa_short_conv(const float* x, const float* w, int taps, const float* state, const int* slots, const int* token_row,
-                              const int* positions, const int* row_start, void* out, int out_code, int n, int width, hipStream_t stream) {
+LSA_EXPORT int lsa_short_conv(const float* x, const float* w, int taps, float* state, const int* slots, const int* token_row,
+                              const int* positions, const int* row_start, void* out, int out_code, int n, int width, int keep,
+                              hipStream_t stream) {
     if (n <= 0) return 0;
     if (taps < 1 || (taps > 1 && (state == nullptr || slots == nullptr))) return -1;
-#define LSA_LAUNCH(O, V) short_conv_kernel<O, V><<<n, 256, 0, stream>>>(x, w, taps, state, slots, token_row, positions, row_start, (O*)out, width)
+#define LSA_LAUNCH(O, V) short_conv_kernel<O, V><<<n, 256, 0, stream>>>(x, w, taps, state, slots, token_row, positions, row_start, (O*)out, width, keep)
     if (width % 4 == 0) { if (out_code) LSA_LAUNCH(bf16_t, 4); else LSA_LAUNCH(float, 4); }
     else { if (out_code) LSA_LAUNCH(bf16_t, 1); else LSA_LAUNCH(float, 1); }
 #undef LSA_LAUNCH

@@ -27,7 +27,7 @@ _SIGNATURES = {
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P, _P],
     "lsa_embedding_norm": [c_int, _P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_norm_rows": [_P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
-    "lsa_short_conv": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_short_conv": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
     "lsa_short_conv_keep": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_scaled_norm_add": [_P, _P, c_int, _P, _P, c_float, _P, _P, c_int, _P, c_long, c_int, _P, c_int, c_int, _P],
     "lsa_latent_prepare": [c_int, _P, c_long, _P, _P, c_float, _P, c_int, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int,

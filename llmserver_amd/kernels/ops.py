@@ -805,8 +805,10 @@ class HipOps(KernelNamespace):
         _launched(self._part_library("stream").lsa_norm_rows(_ptr(x), _ptr(rows), _ptr(weight), float(eps), _ptr(out), _code(out), n_out,
                                                              width, _stream()), "norm_rows")
 
-    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out):
+    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out, keep=False):
         n, width = x.shape
+        if keep and n != row_start.shape[0]:
+            raise ValueError("the state moves on inside this kernel only in steps of one token per row")
         taps = weight.shape[1]
         _check(x, "x", torch.float32)
         _check(weight, "weight", torch.float32, (width, taps))
@@ -821,7 +823,7 @@ class HipOps(KernelNamespace):
             _check(state_slots, "state_slots", torch.int32, (row_start.shape[0],))
         _launched(self._part_library("stream").lsa_short_conv(
             _ptr(x), _ptr(weight), taps, _ptr(state) if taps > 1 else None, _ptr(state_slots) if taps > 1 else None, _ptr(token_row),
-            _ptr(positions), _ptr(row_start), _ptr(out), _code(out), n, width, _stream()), "short_conv")
+            _ptr(positions), _ptr(row_start), _ptr(out), _code(out), n, width, 1 if keep else 0, _stream()), "short_conv")
 
     def short_conv_keep(self, x, state, state_slots, row_start, row_len, row_ctx):
         n, width = x.shape

@@ -174,7 +174,10 @@ class PostNormBlock(Block):
             return out, None
         rounded = None if wide else ctx.empty(x.shape)
         ops.scaled_norm_add(x, mixed, self.mixer_norm.weight, self.scale1, self.mixer_norm.eps, out, rounded=rounded)
-        fed = self.ffn.forward(out if wide else rounded, ctx)
+        if getattr(self.ffn, "reads_stream", False):
+            fed = self.ffn.forward(out if wide else rounded, ctx, stream=out)
+        else:
+            fed = self.ffn.forward(out if wide else rounded, ctx)
         result = ctx.empty(x.shape, dtype=torch.float32)
         ops.scaled_norm_add(out, fed, self.ffn_norm.weight, self.scale2, self.ffn_norm.eps, result, **after)
         return result, None

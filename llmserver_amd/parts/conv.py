@@ -31,7 +31,9 @@ class ShortConvolution(Part):
         """``x [T, W]`` float32 -> ``x + conv(x)`` in the compute type; ``state [slots, taps - 1, W]`` is read, then
         brought up to date with this step's inputs."""
         out = ctx.empty(x.shape)
-        ctx.ops.short_conv(x, self.weight, state, ctx.state_slots, ctx.token_row, ctx.positions, ctx.row_start, out)
-        if state is not None:
+        single = ctx.n_tokens == ctx.n_rows         # one token a row: a row's state is one workgroup's, which moves it on itself
+        ctx.ops.short_conv(x, self.weight, state, ctx.state_slots, ctx.token_row, ctx.positions, ctx.row_start, out,
+                           keep=single and state is not None)
+        if state is not None and not single:
             ctx.ops.short_conv_keep(x, state, ctx.state_slots, ctx.row_start, ctx.row_len, ctx.row_ctx)
         return out

@@ -13,6 +13,8 @@ from .base import VECTOR, FeedForward, ParamSpec
 
 
 class RoutedExperts(FeedForward):
+    reads_stream = True       # forward takes ``stream=``: the 32-bit rows that ``x`` was rounded from, for the router
+
     def __init__(self, width: int, intermediate: int, experts: int, top: int, router: str = "router", expert: str = "e{}",
                  pieces=("gate", "up", "down")):
         if not 1 <= top <= experts:
@@ -51,13 +53,14 @@ class RoutedExperts(FeedForward):
         self.down = torch.stack([self._parts[down] for _, _, _, down in names]).contiguous()
         self._parts.clear()
 
-    def forward(self, x, ctx):
-        """``x [T, W]`` in the compute type -> float32 ``[T, W]``."""
+    def forward(self, x, ctx, stream=None):
+        """``x [T, W]`` in the compute type -> float32 ``[T, W]``.  ``stream``: the same rows in 32-bit, if the caller
+        has them (the router's logits are 32-bit either way; from these they need no widening first)."""
         ops = ctx.ops
         n = x.shape[0]
         chosen = ctx.empty((n, self.top), dtype=torch.int32)
         weights = ctx.empty((n, self.top), dtype=torch.float32)
-        ops.route_experts(x, self.router, self.top, chosen, weights)
+        ops.route_experts(x if stream is None else stream, self.router, self.top, chosen, weights)
         out = ctx.empty((n, self.width), dtype=torch.float32)
         if ops.experts_sorted(x, self.gate_up, self.down, chosen, weights, out):       # many tokens: pairs sorted by expert
             return out

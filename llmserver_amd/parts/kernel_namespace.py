@@ -59,10 +59,11 @@ class KernelNamespace:
         """``out = rmsnorm(x[rows]) * weight`` for a float32 ``x``; ``rows`` int32 or None (all); ``out`` of any type."""
         raise NotImplementedError
 
-    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out):
+    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out, keep=False):
         """``out = x + conv(x)``: a causal convolution over each request's tokens on every channel, ``weight [W, taps]``,
         tap ``j`` on the token ``taps - 1 - j`` places back; tokens before the step's come from ``state [slots, taps - 1,
-        W]`` (a request's last inputs, oldest first), tokens before the sequence are zeros.  ``x`` float32."""
+        W]`` (a request's last inputs, oldest first), tokens before the sequence are zeros.  ``x`` float32.  ``keep``
+        (steps of one token per row only): the state also moves on by the step's token, as :meth:`short_conv_keep` would do."""
         raise NotImplementedError
 
     def short_conv_keep(self, x, state, state_slots, row_start, row_len, row_ctx):

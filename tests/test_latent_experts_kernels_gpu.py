@@ -70,8 +70,9 @@ def test_short_convolution_with_state_over_steps(ops, dtype, taps):
         x = torch.randn(sum(lengths), width, device="cuda")
         outs = [torch.empty(sum(lengths), width, device="cuda", dtype=dtype) for _ in range(2)]
         for which, state, out in ((ops, states[0], outs[0]), (twin, states[1], outs[1])):
-            which.short_conv(x, weight, state, slot_of, token_row, positions, row_start, out)
-            if state is not None:
+            single = max(lengths) == 1 and state is not None       # one token a row: the kernel may move the state on itself
+            which.short_conv(x, weight, state, slot_of, token_row, positions, row_start, out, keep=single)
+            if state is not None and not single:
                 which.short_conv_keep(x, state, slot_of, row_start, row_len, row_ctx)
         close(outs[0], outs[1], dtype, f"short_conv {lengths}")
         if taps > 1:
@@ -173,7 +174,7 @@ def test_routed_experts(ops, dtype, experts, top, width, inter):
     close(results[0][3], results[1][3], dtype, "out")
 
 
-@pytest.mark.parametrize("experts, top, width, inter, tokens", [(5, 2, 64, 32, 40), (12, 3, 96, 160, 333), (70, 6, 256, 96, 200), (3, 1, 32, 64, 700)])
+@pytest.mark.parametrize("experts, top, width, inter, tokens", [(5, 2, 64, 32, 40), (12, 3, 96, 160, 333), (70, 6, 256, 96, 200), (70, 6, 256, 96, 100), (40, 2, 64, 128, 90), (3, 1, 32, 64, 700)])
 def test_sorted_expert_products_equal_the_per_pair_ones(ops, experts, top, width, inter, tokens):
     """Many tokens: the pairs sorted by expert and multiplied tile by tile give what every pair alone gives."""
     print(f"sorted experts {experts} {top} {width} {inter} {tokens}", flush=True)

@@ -194,7 +194,7 @@ class TorchOps(KernelNamespace):
         picked = x if rows is None else x[rows.long()]
         out.copy_((self._rms(picked.float(), eps) * weight).to(out.dtype))
 
-    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out):
+    def short_conv(self, x, weight, state, state_slots, token_row, positions, row_start, out, keep=False):
         taps = weight.shape[1]
         result = x.clone()
         for t in range(x.shape[0]):
@@ -211,6 +211,11 @@ class TorchOps(KernelNamespace):
                     value = state[int(state_slots[row]), taps - 1 - (first - place)]
                 result[t] += weight[:, j] * value
         out.copy_(result.to(out.dtype))
+        if keep:
+            assert x.shape[0] == len(row_start)
+            for t in range(x.shape[0]):
+                slot = int(state_slots[int(token_row[t])])
+                state[slot] = torch.cat([state[slot, 1:], x[t:t + 1]], dim=0)
 
     def short_conv_keep(self, x, state, state_slots, row_start, row_len, row_ctx):
         kept = state.shape[1]
