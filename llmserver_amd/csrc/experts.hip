@@ -53,6 +53,27 @@ __device__ inline void wave_dot2(const T* __restrict__ w0, const T* __restrict__
     r1 = wave_sum(a1);
 }
 
+// Router logits for steps of few tokens, where a library product would be a launch of 11 us for a few thousand
+// multiplications: grid (tokens, experts / 4), a wavefront per expert, float32 throughout.
+__global__ __launch_bounds__(256) void route_logits_kernel(const float* __restrict__ x, const float* __restrict__ router,
+                                                           float* __restrict__ logits, int experts, int width) {
+    const int lane = threadIdx.x & 63, e = blockIdx.y * 4 + (threadIdx.x >> 6), t = blockIdx.x;
+    if (e >= experts) return;
+    const float* r = router + (size_t)e * width;
+    const float* row = x + (size_t)t * width;
+    float acc = 0.f;
+    if (width % 4 == 0) {
+        for (int i = lane * 4; i < width; i += 256) {
+            const float4 a = *reinterpret_cast<const float4*>(r + i), b = *reinterpret_cast<const float4*>(row + i);
+            acc += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+        }
+    } else {
+        for (int i = lane; i < width; i += 64) acc += r[i] * row[i];
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) logits[(size_t)t * experts + e] = acc;
+}
+
 // One wavefront per token: the `top` largest of the token's float32 logits (the lowest index among equal ones) and
 // their softmax.  The logits themselves are a float32 matrix product made before this kernel.  A lane keeps the logits
 // of experts lane, lane + 64, ... in LDS (its own entries only: nothing crosses lanes through LDS), and every lane ends
@@ -179,6 +200,12 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
         acc = wave_sum(acc);
         if (lane == 0) out[(size_t)t * width + c] = acc;
     }
+}
+
+LSA_EXPORT int lsa_route_logits(const float* x, const float* router, float* logits, int n, int experts, int width, hipStream_t stream) {
+    if (n <= 0) return 0;
+    route_logits_kernel<<<dim3(n, (experts + 3) / 4), 256, 0, stream>>>(x, router, logits, experts, width);
+    LSA_LAUNCH_CHECK();
 }
 
 LSA_EXPORT int lsa_route_top(const float* logits, int experts, int top, int* chosen, float* weights, int n, hipStream_t stream) {

@@ -30,9 +30,10 @@ _SIGNATURES = {
     "lsa_short_conv": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
     "lsa_short_conv_keep": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_scaled_norm_add": [_P, _P, c_int, _P, _P, c_float, _P, _P, c_int, _P, c_long, c_int, _P, c_int, c_int, _P],
-    "lsa_latent_prepare": [c_int, _P, c_long, _P, _P, c_float, _P, c_int, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int,
+    "lsa_latent_prepare": [c_int, _P, c_long, _P, _P, _P, c_float, _P, c_int, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int,
                            c_int, c_int, c_int, c_int, _P],
-    "lsa_gate_heads": [c_int, _P, _P, c_long, c_int, _P, c_int, c_int, c_int, _P],
+    "lsa_gate_heads": [c_int, _P, _P, _P, c_int, c_int, _P, c_long, c_int, _P, c_int, c_int, c_int, _P],
+    "lsa_route_logits": [_P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_route_top": [_P, c_int, c_int, _P, _P, c_int, _P],
     "lsa_experts_gate_up": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_experts_tile_rows": [],

@@ -857,13 +857,23 @@ class HipOps(KernelNamespace):
             _code(rounded) if rounded is not None else 0, _ptr(history), n * width, int(before), _ptr(mix), n, width, _stream()),
             "scaled_norm_add")
 
+    LATENT_FEW_ROWS = 16      # up to this many tokens the per-head products of the latent attention are made inside its kernels
+
+    def latent_products_inside(self, n_tokens: int) -> bool:
+        return 0 < n_tokens <= self.LATENT_FEW_ROWS
+
     def latent_prepare(self, proj, q_latent, norm_weight, eps, cos_sin, keys, values, table, token_row, positions, page_size,
-                       out_q, n_heads, dim, rot_dim, rank, write_cache=True):
+                       out_q, n_heads, dim, rot_dim, rank, write_cache=True, up_keys=None):
         n = proj.shape[0]
         _check(proj, "proj")
         if proj.shape[1] < n_heads * (dim + rot_dim) + rank + rot_dim:
             raise ValueError(f"proj has {proj.shape[1]} columns, queries and the latent need {n_heads * (dim + rot_dim) + rank + rot_dim}")
-        _check(q_latent, "q_latent", proj.dtype, (n_heads, n, rank))
+        if (q_latent is None) == (up_keys is None):
+            raise ValueError("the queries' latent part comes as q_latent or is multiplied here with up_keys: exactly one of them")
+        if q_latent is not None:
+            _check(q_latent, "q_latent", proj.dtype, (n_heads, n, rank))
+        else:
+            _check(up_keys, "up_keys", proj.dtype, (n_heads, dim, rank))
         _check(norm_weight, "norm_weight", torch.float32, (rank,))
         pairs = cos_sin.shape[1] // 2
         _check(cos_sin, "cos_sin", torch.float32, (n, 2 * pairs))
@@ -879,19 +889,31 @@ class HipOps(KernelNamespace):
         _check(positions, "positions", torch.int32, (n,))
         _check(out_q, "out_q", proj.dtype, (n, n_heads * row_width))
         _launched(self._part_library("latent").lsa_latent_prepare(
-            _code(proj), _ptr(proj), proj.shape[1], _ptr(q_latent), _ptr(norm_weight), float(eps), _ptr(cos_sin), pairs, _ptr(keys),
-            _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions), page_size, _ptr(out_q), n_heads, dim, rot_dim,
-            rank, row_width, 1 if write_cache else 0, n, _stream()), "latent_prepare")
+            _code(proj), _ptr(proj), proj.shape[1], _ptr(q_latent), _ptr(up_keys), _ptr(norm_weight), float(eps), _ptr(cos_sin), pairs,
+            _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions), page_size, _ptr(out_q), n_heads, dim,
+            rot_dim, rank, row_width, 1 if write_cache else 0, n, _stream()), "latent_prepare")
 
-    def gate_heads(self, y, proj, gate_column, out):
-        heads, n, v = y.shape
-        _check(y, "y", out.dtype)
+    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None):
         _check(proj, "proj", out.dtype)
-        _check(out, "out", None, (n, heads * v))
-        if proj.shape[0] != n or gate_column + heads > proj.shape[1]:
-            raise ValueError(f"gates of {heads} heads from column {gate_column} do not lie in proj {tuple(proj.shape)}")
-        _launched(self._part_library("latent").lsa_gate_heads(_code(out), _ptr(y), _ptr(proj), proj.shape[1], int(gate_column), _ptr(out),
-                                                              heads, v, n, _stream()), "gate_heads")
+        _check(out, "out")
+        n = out.shape[0]
+        if (y is None) == (up_values is None):
+            raise ValueError("the heads' values come as y or are multiplied here from mixed with up_values: exactly one of them")
+        if y is not None:
+            heads, _, v = y.shape
+            _check(y, "y", out.dtype, (heads, n, v))
+            rank = row_width = 0
+        else:
+            heads, rank, v = up_values.shape
+            _check(up_values, "up_values", out.dtype)
+            _check(mixed, "mixed", out.dtype)
+            row_width = mixed.shape[1] // heads
+            if mixed.shape != (n, heads * row_width) or rank > row_width:
+                raise ValueError(f"mixed {tuple(mixed.shape)} does not hold {heads} rows of at least {rank} a token")
+        if tuple(out.shape) != (n, heads * v) or proj.shape[0] != n or gate_column + heads > proj.shape[1]:
+            raise ValueError(f"gates of {heads} heads from column {gate_column} of proj {tuple(proj.shape)} for an output of {tuple(out.shape)}")
+        _launched(self._part_library("latent").lsa_gate_heads(_code(out), _ptr(y), _ptr(mixed), _ptr(up_values), rank, row_width, _ptr(proj),
+                                                              proj.shape[1], int(gate_column), _ptr(out), heads, v, n, _stream()), "gate_heads")
 
     def route_experts(self, x, router, top, chosen, weights):
         """The logits are a float32 product of the library (no reduced-precision mode), the choice and the softmax a kernel."""
@@ -903,7 +925,13 @@ class HipOps(KernelNamespace):
         _check(weights, "weights", torch.float32, (n, top))
         if not 1 <= top <= experts or experts > 3072:
             raise ValueError(f"the router kernel chooses 1 to {min(experts, 3072)} of up to 3072 experts, asked for {top} of {experts}")
-        logits = torch.mm(x if x.dtype == torch.float32 else x.float(), router.t())
+        wide = x if x.dtype == torch.float32 else x.float()
+        if n <= self.LATENT_FEW_ROWS:          # few tokens: a kernel of a few microseconds instead of a library call
+            logits = torch.empty((n, experts), device=x.device, dtype=torch.float32)
+            _launched(self._part_library("experts").lsa_route_logits(_ptr(wide), _ptr(router), _ptr(logits), n, experts, width, _stream()),
+                      "route_logits")
+        else:
+            logits = torch.mm(wide, router.t())
         _launched(self._part_library("experts").lsa_route_top(_ptr(logits), experts, top, _ptr(chosen), _ptr(weights), n, _stream()),
                   "route_top")
 

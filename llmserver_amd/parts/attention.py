@@ -506,7 +506,7 @@ class GQAttention(Mixer):
         self.o.finalize()
 
     def plan_key(self):
-        return ("paged_attention", self.group_size, self.n_kv_heads, self.window)
+        return ("paged_attention", self.group_size, self.n_kv_heads, self.window, self.head_dim)
 
     def graph_shape(self, rows: int, longest_context: int):
         return "short contexts" if longest_context <= SHORT_CONTEXT else None

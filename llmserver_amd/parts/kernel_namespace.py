@@ -78,16 +78,18 @@ class KernelNamespace:
 
     # Attention over a shared low-rank latent.
     def latent_prepare(self, proj, q_latent, norm_weight, eps, cos_sin, keys, values, table, token_row, positions, page_size,
-                       out_q, n_heads, dim, rot_dim, rank, write_cache=True):
+                       out_q, n_heads, dim, rot_dim, rank, write_cache=True, up_keys=None):
         """``proj [T, n_heads * (dim + rot_dim) + rank + rot_dim + ...]``: per head ``dim`` plain and ``rot_dim`` rotated
         query dimensions, then the token's ``rank`` latent dimensions and its ``rot_dim`` shared rotated key dimensions.
         Writes a cache row ``[rmsnorm(latent) * norm_weight, rotate(key part), zeros]`` of every token as its key and,
         transposed, as its value, and ``out_q [T, n_heads * D]`` with per head ``[q_latent[h, t], rotate(q's rotated part),
-        zeros]``.  ``cos_sin [T, 2 * pairs]``: neighbouring dimensions (2i, 2i+1) of the first ``2 * pairs`` rotated ones turn."""
+        zeros]``.  ``cos_sin [T, 2 * pairs]``: neighbouring dimensions (2i, 2i+1) of the first ``2 * pairs`` rotated ones turn.
+        ``q_latent`` None and ``up_keys [heads, dim, rank]`` given: ``q_latent[h, t] = q_plain[t, h] @ up_keys[h]`` is made here."""
         raise NotImplementedError
 
-    def gate_heads(self, y, proj, gate_column, out):
-        """``out[t, h * v + j] = y[h, t, j] * sigmoid(proj[t, gate_column + h])``."""
+    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None):
+        """``out[t, h * v + j] = y[h, t, j] * sigmoid(proj[t, gate_column + h])`` (``gate_column`` < 0: no gate).  ``y`` None and
+        ``mixed [T, heads * row]``, ``up_values [heads, rank, v]`` given: ``y[h, t] = mixed[t, h, :rank] @ up_values[h]`` is made here."""
         raise NotImplementedError
 
     # Routed experts.
@@ -107,6 +109,11 @@ class KernelNamespace:
         raise NotImplementedError
 
     # -- what a namespace may offer; the answers here mean "not offered" --------------------------------------------
+    def latent_products_inside(self, n_tokens: int) -> bool:
+        """Whether, for a step of this many tokens, :meth:`latent_prepare` and :meth:`gate_heads` should make the per-head
+        products themselves (``up_keys=`` / ``up_values=``) instead of getting them from batched products made before."""
+        return False
+
     def experts_sorted(self, x, gate_up, down, chosen, weights, out) -> bool:
         """Both products of the routed experts and the weighted sum for all of the step's tokens at once, the (token,
         expert) pairs sorted by expert so that an expert's matrices are read once per tile of pairs: ``out`` as

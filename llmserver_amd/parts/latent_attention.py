@@ -102,7 +102,8 @@ class LatentAttention(Mixer):
         self._up_keys = self._up_values = None
 
     def plan_key(self):
-        return ("paged_attention", self.n_heads, 1, None)
+        # (the row's width is part of it: the plan is cut for the kernels of that head size)
+        return ("paged_attention", self.n_heads, 1, None, self.row)
 
     def graph_shape(self, rows: int, longest_context: int):
         return "short contexts" if longest_context <= SHORT_CONTEXT else None
@@ -124,20 +125,26 @@ class LatentAttention(Mixer):
         n = x.shape[0]
         proj = self.proj.forward(x, ctx)                                        # [T, q | latent, key part | gates]
         per_head = self.dim + self.rot_dim
-        q_plain = proj[:, :self.q_width].view(n, self.n_heads, per_head)[:, :, :self.dim].transpose(0, 1)
-        q_latent = torch.bmm(q_plain, self.up_keys)                            # [heads, T, rank]
+        inside = ops.latent_products_inside(n)      # few tokens: the per-head products are made inside the kernels around attention
+        q_latent = None
+        if not inside:
+            q_plain = proj[:, :self.q_width].view(n, self.n_heads, per_head)[:, :, :self.dim].transpose(0, 1)
+            q_latent = torch.bmm(q_plain, self.up_keys)                        # [heads, T, rank]
         table = ctx.block_table(cache.group)
         q = ctx.empty((n, self.n_heads * self.row))
         ops.latent_prepare(proj, q_latent, self.down_norm_weight, self.norm_eps, self.position.cos_sin(ctx), cache.keys, cache.values,
                            table, ctx.token_row, ctx.positions, cache.page_size, q, self.n_heads, self.dim, self.rot_dim, self.rank,
-                           cache.writable)
+                           cache.writable, **({"up_keys": self.up_keys} if inside else {}))
         mixed = ctx.empty((n, self.n_heads * self.row))
         extra = {"sinks": self.sinks} if self.sinks is not None else {}
         ops.paged_attention(q, mixed, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
                             ctx.get_plan(self.plan_key()), self.scale, None, cache.page_size, self.n_heads, 1, self.row, ctx, **extra)
-        latent = mixed.view(n, self.n_heads, self.row)[:, :, :self.rank].transpose(0, 1)
-        up = torch.bmm(latent, self.up_values)                                  # [heads, T, value_dim]
         gated = ctx.empty((n, self.n_heads * self.value_dim))
         # (without gates the same kernel only brings the heads back beside each other: a gate column of -1 says so)
-        ops.gate_heads(up, proj, self.q_width + self.rank + self.rot_dim if self.names.gate is not None else -1, gated)
+        gate_column = self.q_width + self.rank + self.rot_dim if self.names.gate is not None else -1
+        if inside:
+            ops.gate_heads(None, proj, gate_column, gated, mixed=mixed, up_values=self.up_values)
+        else:
+            latent = mixed.view(n, self.n_heads, self.row)[:, :, :self.rank].transpose(0, 1)
+            ops.gate_heads(torch.bmm(latent, self.up_values), proj, gate_column, gated)      # [heads, T, value_dim]
         return self.o.forward(gated, ctx)

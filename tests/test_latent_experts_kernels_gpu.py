@@ -131,8 +131,17 @@ def test_latent_prepare_and_gate_heads(ops, dtype, heads, dim, rot_dim, rank, pa
         gated, plain = torch.empty(n, heads * 12, device="cuda", dtype=dtype), torch.empty(n, heads * 12, device="cuda", dtype=dtype)
         which.gate_heads(y, proj, heads * (dim + rot_dim) + rank + rot_dim, gated)
         which.gate_heads(y, proj, -1, plain)
-        results.append((keys, values, out_q, gated, plain))
-    for got, want, what in zip(results[0], results[1], ("keys", "values", "q", "gated", "ungated")):
+        # the same with the per-head products made inside the kernels (steps of few tokens go this way)
+        generator = torch.Generator(device="cuda").manual_seed(4)
+        up_keys = (torch.randn(heads, dim, rank, device="cuda", generator=generator) / dim ** 0.5).to(dtype)
+        up_values = (torch.randn(heads, rank, 12, device="cuda", generator=generator) / rank ** 0.5).to(dtype)
+        inside_q = torch.empty(n, heads * row_width, device="cuda", dtype=dtype)
+        which.latent_prepare(proj, None, norm_weight, 1e-5, cos_sin, keys, values, table, token_row, positions, page_size, inside_q,
+                             heads, dim, rot_dim, rank, False, up_keys=up_keys)
+        inside_gated = torch.empty(n, heads * 12, device="cuda", dtype=dtype)
+        which.gate_heads(None, proj, heads * (dim + rot_dim) + rank + rot_dim, inside_gated, mixed=out_q, up_values=up_values)
+        results.append((keys, values, out_q, gated, plain, inside_q, inside_gated))
+    for got, want, what in zip(results[0], results[1], ("keys", "values", "q", "gated", "ungated", "q made inside", "gated made inside")):
         close(got, want, dtype, what)
     assert torch.equal(results[0][0].transpose(2, 3)[results[0][0].transpose(2, 3) != 7], results[0][1][results[0][1] != 7])
 

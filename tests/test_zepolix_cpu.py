@@ -273,3 +273,15 @@ def test_greedy_generation_through_the_entry_point_equals_the_oracles():
     got = generate(model_folder("ZB"), prompts, max_new_tokens=7, dtype="float32", device="cpu", block_size=8, num_blocks=26,
                    max_batch_size=3, max_num_batched_tokens=24, prefill_chunk_size=16, ops=TorchOps())
     assert got == expected
+
+
+def test_the_per_head_products_made_inside_the_kernels_give_the_same(tmp_path):
+    """Steps of few tokens let the kernels around attention multiply with the heads' matrices themselves; the twins of
+    that dataflow match the oracle like the batched products do."""
+    ops = TorchOps()
+    ops.inside = True
+    requests = requests_of("ZB", (40, 9))
+    steps = traces.tail_decoded(requests, 12)
+    runner = make_runner(model_folder("ZB"), "float32", traces.peak_tokens(steps), 8, device="cpu", ops=ops)
+    replay(runner, traces.to_lines(steps).splitlines(), str(tmp_path), io.StringIO())
+    check("ZB", traces.collect(steps, str(tmp_path), CASES["ZB"][0]["vocab"]), requests)

@@ -38,11 +38,15 @@ ZB = config(130, 64, 1e-6, 4, [layer(mixer(5, 12, 8, 10, 40, base=500.0, dims=4)
 ZC = config(61, 40, 3e-4, 0, [layer(mixer(17, 4, 2, 3, 12), experts(7, 9, 3)), layer(mixer(1, 24, 8, 40, 24), experts(16, 2, 1))])
 ZD = config(200, 72, 1e-5, 2, [layer(mixer(6, 10, 6, 12, 58, base=2e4), experts(24, 6, 2)) for _ in range(2)])
 ZE = config(50, 32, 1e-5, 5, [layer(mixer(2, 8, 8, 8, 8, base=100.0), experts(8, 2, 2))])
+# Two layers with the same number of heads whose cache rows differ in width (two groups of pages, two attention plans), the
+# second as wide as the kernels' widest head with the smaller tile shape.
+ZF = config(77, 56, 2e-5, 3, [layer(mixer(4, 8, 4, 8, 24), experts(16, 4, 2)), layer(mixer(4, 12, 10, 6, 130, base=3000.0), experts(8, 3, 1))])
 
 INIT = RandomInit(seed=3, std=0.15, norm_noise=0.3, bias_std=0.2)
 CASES = {"ZA": (ZA, INIT, 16), "ZB": (ZB, RandomInit(seed=8, std=0.12, norm_noise=0.2, bias_std=0.3), 8),
          "ZC": (ZC, RandomInit(seed=21, std=0.2, norm_noise=0.25, bias_std=0.1), 4), "ZD": (ZD, INIT, 16),
-         "ZE": (ZE, RandomInit(seed=2, std=0.25, norm_noise=0.3, bias_std=0.2), 8)}
+         "ZE": (ZE, RandomInit(seed=2, std=0.25, norm_noise=0.3, bias_std=0.2), 8),
+         "ZF": (ZF, RandomInit(seed=13, std=0.12, norm_noise=0.2, bias_std=0.2), 16)}
 
 _FOLDERS = {}
 

@@ -242,10 +242,17 @@ class TorchOps(KernelNamespace):
             rounded.copy_(s.to(rounded.dtype))
 
     # -- attention over a shared latent ------------------------------------------------------------------
+    inside = False          # True: the parts are told to let latent_prepare and gate_heads make the per-head products
+
+    def latent_products_inside(self, n_tokens):
+        return self.inside
+
     def latent_prepare(self, proj, q_latent, norm_weight, eps, cos_sin, keys, values, table, token_row, positions, page_size,
-                       out_q, n_heads, dim, rot_dim, rank, write_cache=True):
+                       out_q, n_heads, dim, rot_dim, rank, write_cache=True, up_keys=None):
         n, width = proj.shape[0], keys.shape[-1]
         q = proj[:, :n_heads * (dim + rot_dim)].float().view(n, n_heads, dim + rot_dim)
+        if q_latent is None:
+            q_latent = torch.einsum("thd,hdr->htr", q[..., :dim], up_keys.float())
         down = proj[:, n_heads * (dim + rot_dim):n_heads * (dim + rot_dim) + rank + rot_dim].float()
         pairs = cos_sin.shape[1] // 2
         cos, sin = cos_sin[:, :pairs], cos_sin[:, pairs:]
@@ -271,7 +278,11 @@ class TorchOps(KernelNamespace):
         keys[pages, 0, slots, :] = row.to(keys.dtype)
         values[pages, 0, :, slots] = row.to(values.dtype)
 
-    def gate_heads(self, y, proj, gate_column, out):
+    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None):
+        if y is None:
+            heads, rank, _ = up_values.shape
+            rows = mixed.float().view(mixed.shape[0], heads, -1)[:, :, :rank]
+            y = torch.einsum("thr,hrv->htv", rows, up_values.float())
         heads, n, v = y.shape
         gate = torch.sigmoid(proj[:, gate_column:gate_column + heads].float()) if gate_column >= 0 else torch.ones(n, heads, device=y.device)
         out.copy_((y.float().transpose(0, 1) * gate[..., None]).reshape(n, heads * v).to(out.dtype))
