@@ -147,7 +147,7 @@ def test_latent_prepare_and_gate_heads(ops, dtype, heads, dim, rot_dim, rank, pa
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("experts, top, width, inter", [(5, 1, 24, 10), (12, 2, 100, 36), (70, 6, 256, 64), (4, 4, 30, 7)])
+@pytest.mark.parametrize("experts, top, width, inter", [(5, 1, 24, 10), (12, 2, 100, 36), (70, 6, 320, 64), (4, 4, 30, 7)])
 def test_routed_experts(ops, dtype, experts, top, width, inter):
     print(f"experts {dtype} {experts} {top} {width} {inter}", flush=True)
     twin, n = TorchOps(), 13
@@ -183,7 +183,7 @@ def test_routed_experts(ops, dtype, experts, top, width, inter):
     close(results[0][3], results[1][3], dtype, "out")
 
 
-@pytest.mark.parametrize("experts, top, width, inter, tokens", [(5, 2, 64, 32, 40), (12, 3, 96, 160, 333), (70, 6, 256, 96, 200), (70, 6, 256, 96, 100), (40, 2, 64, 128, 90), (3, 1, 32, 64, 700)])
+@pytest.mark.parametrize("experts, top, width, inter, tokens", [(5, 2, 64, 32, 40), (12, 3, 96, 160, 333), (70, 6, 192, 96, 200), (70, 6, 192, 96, 100), (40, 2, 64, 128, 90), (3, 1, 32, 64, 700)])
 def test_sorted_expert_products_equal_the_per_pair_ones(ops, experts, top, width, inter, tokens):
     """Many tokens: the pairs sorted by expert and multiplied tile by tile give what every pair alone gives."""
     print(f"sorted experts {experts} {top} {width} {inter} {tokens}", flush=True)
