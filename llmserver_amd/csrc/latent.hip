@@ -15,57 +15,64 @@ __device__ inline float turned(const T* __restrict__ v, int e, const float* __re
     return (e & 1) ? w * c + u * s : u * c - w * s;
 }
 
-// grid (tokens, heads + 1).  proj row: heads x [dim plain, rot_dim rotated] query dimensions, then the token's `rank`
-// latent dimensions and its rot_dim rotated key dimensions.  Workgroup (t, h < heads) assembles head h's query row
-// [U_h^T q_h, rotate(p_h), zeros]; the first part comes from `q_latent` [heads][tokens][rank] (a batched product made
-// before) or, where `up_keys` [heads][dim][rank] is given (steps of few tokens, where that product would be a launch of
-// its own for a few thousand multiplications), is multiplied here.  Workgroup (t, heads) writes the token's cache row.
+// grid (tokens, heads + 1, pieces of 64 of a row).  proj row: heads x [dim plain, rot_dim rotated] query dimensions, then
+// the token's `rank` latent dimensions and its rot_dim rotated key dimensions.  Workgroups (t, h < heads, piece) assemble
+// head h's query row [U_h^T q_h, rotate(p_h), zeros], 64 elements each; the first part comes from `q_latent`
+// [heads][tokens][rank] (a batched product made before) or, where `up_keys` [heads][dim][rank] is given (steps of few tokens,
+// where that product would be a launch of its own for a few thousand multiplications), is multiplied here: a lane owns an
+// element, the workgroup's wavefronts share the rows of the matrix between them and add their sums up in LDS.
+// Workgroup (t, heads, 0) writes the token's cache row.
 template <typename T>
-__global__ __launch_bounds__(256) void latent_prepare_kernel(
+__global__ void latent_prepare_kernel(
     const T* __restrict__ proj, long proj_stride, const T* __restrict__ q_latent, const T* __restrict__ up_keys,
     const float* __restrict__ norm_weight, float eps,
     const float* __restrict__ cos_sin, int pairs, T* __restrict__ keys, T* __restrict__ values, const int* __restrict__ table,
     int table_stride, const int* __restrict__ token_row, const int* __restrict__ positions, int page_size, T* __restrict__ out_q,
     int heads, int dim, int rot_dim, int rank, int row_width, int write_cache, int n_tokens) {
-    extern __shared__ float q_lds[];                // dim floats, where the product is made here
     __shared__ float scratch[16];
+    __shared__ float partial[4][64];
     const int t = blockIdx.x, head = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const T* mine = proj + (size_t)t * proj_stride;
     const float* cs = cos_sin + (size_t)t * 2 * pairs;
     const int per_head = dim + rot_dim;
     if (head < heads) {
         const T* qh = mine + head * per_head;
-        T* q = out_q + ((size_t)t * heads + head) * row_width;
-        if (up_keys) {
-            for (int d = threadIdx.x; d < dim; d += blockDim.x) q_lds[d] = (float)qh[d];
-            __syncthreads();
-        }
-        for (int e = threadIdx.x; e < row_width; e += blockDim.x) {
-            float v = 0.f;
-            if (e < rank) {
-                if (up_keys) {
-                    // (eight loads under way at a time: the rows of the matrix are independent of one another)
-                    const T* u = up_keys + (size_t)head * dim * rank + e;
-                    int d = 0;
-                    for (; d + 8 <= dim; d += 8) {
-                        float w[8];
-#pragma unroll
-                        for (int k = 0; k < 8; ++k) w[k] = (float)u[(size_t)(d + k) * rank];
-#pragma unroll
-                        for (int k = 0; k < 8; ++k) v += q_lds[d + k] * w[k];
-                    }
-                    for (; d < dim; ++d) v += q_lds[d] * (float)u[(size_t)d * rank];
-                } else {
-                    v = (float)q_latent[((size_t)head * n_tokens + t) * rank + e];
-                }
-            } else if (e < rank + rot_dim) {
-                v = turned(qh + dim, e - rank, cs, pairs);
+        if (!up_keys) {                 // nothing to multiply: one workgroup assembles the whole row
+            for (int e = threadIdx.x; e < row_width; e += blockDim.x) {
+                float v = 0.f;
+                if (e < rank) v = (float)q_latent[((size_t)head * n_tokens + t) * rank + e];
+                else if (e < rank + rot_dim) v = turned(qh + dim, e - rank, cs, pairs);
+                out_q[((size_t)t * heads + head) * row_width + e] = (T)v;
             }
-            q[e] = (T)v;
+            return;
         }
+        const int e = blockIdx.z * 64 + lane;
+        float v = 0.f;
+        if (e < rank) {
+            const int share = (dim + waves - 1) / waves, d0 = wave * share, d1 = min(dim, d0 + share);
+            const T* u = up_keys + (size_t)head * dim * rank + e;
+            int d = d0;
+            for (; d + 8 <= d1; d += 8) {                   // eight rows of the matrix under way at a time
+                float w[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) w[k] = (float)u[(size_t)(d + k) * rank];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) v += (float)qh[d + k] * w[k];
+            }
+            for (; d < d1; ++d) v += (float)qh[d] * (float)u[(size_t)d * rank];
+        }
+        partial[wave][lane] = v;
+        __syncthreads();
+        if (wave) return;
+        v = 0.f;
+        for (int w = 0; w < waves; ++w) v += partial[w][lane];
+        if (e >= row_width) return;
+        if (e >= rank) v = e < rank + rot_dim ? turned(qh + dim, e - rank, cs, pairs) : 0.f;
+        out_q[((size_t)t * heads + head) * row_width + e] = (T)v;
         return;
     }
-    if (!write_cache) return;
+    if (!write_cache || blockIdx.z) return;
     const T* down = mine + (size_t)heads * per_head;
     float sq = 0.f;
     for (int i = threadIdx.x; i < rank; i += blockDim.x) {
@@ -87,41 +94,50 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     }
 }
 
-// grid (tokens, heads): out[t][h * v + j] = y_h[t][j] * sigmoid(proj[t][gate_column + h])   (gate_column < 0: no gate), where
-// y_h[t] comes from `y` [heads][tokens][v] (a batched product made before) or, where `up_values` [heads][rank][v] is given,
-// is the head's weighted latent sum `mixed[t][h][0 .. rank)` (rows of row_width) times that matrix, multiplied here.
+// grid (tokens, heads, pieces of 64 of a head's values): out[t][h * v + j] = y_h[t][j] * sigmoid(proj[t][gate_column + h])
+// (gate_column < 0: no gate), where y_h[t] comes from `y` [heads][tokens][v] (a batched product made before) or, where
+// `up_values` [heads][rank][v] is given, is the head's weighted latent sum `mixed[t][h][0 .. rank)` (rows of row_width) times
+// that matrix, multiplied here as in the kernel above.
 template <typename T>
-__global__ __launch_bounds__(256) void gate_heads_kernel(const T* __restrict__ y, const T* __restrict__ mixed, const T* __restrict__ up_values,
-                                                         int rank, int row_width, const T* __restrict__ proj, long proj_stride,
-                                                         int gate_column, T* __restrict__ out, int heads, int v, int n_tokens) {
-    extern __shared__ float latent_lds[];           // rank floats, where the product is made here
+__global__ void gate_heads_kernel(const T* __restrict__ y, const T* __restrict__ mixed, const T* __restrict__ up_values,
+                                  int rank, int row_width, const T* __restrict__ proj, long proj_stride,
+                                  int gate_column, T* __restrict__ out, int heads, int v, int n_tokens) {
+    __shared__ float partial[4][64];
     const int t = blockIdx.x, head = blockIdx.y;
-    float g = 1.f;
-    if (gate_column >= 0) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + head]));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int j = blockIdx.z * 64 + lane;
+    float value = 0.f;
     if (up_values) {
-        const T* row = mixed + ((size_t)t * heads + head) * row_width;
-        for (int r = threadIdx.x; r < rank; r += blockDim.x) latent_lds[r] = (float)row[r];
-        __syncthreads();
-    }
-    for (int j = threadIdx.x; j < v; j += blockDim.x) {
-        float value;
-        if (up_values) {
+        if (j < v) {
+            const T* row = mixed + ((size_t)t * heads + head) * row_width;
+            const int share = (rank + waves - 1) / waves, r0 = wave * share, r1 = min(rank, r0 + share);
             const T* u = up_values + (size_t)head * rank * v + j;
-            value = 0.f;
-            int r = 0;
-            for (; r + 8 <= rank; r += 8) {
+            int r = r0;
+            for (; r + 8 <= r1; r += 8) {
                 float w[8];
 #pragma unroll
                 for (int k = 0; k < 8; ++k) w[k] = (float)u[(size_t)(r + k) * v];
 #pragma unroll
-                for (int k = 0; k < 8; ++k) value += latent_lds[r + k] * w[k];
+                for (int k = 0; k < 8; ++k) value += (float)row[r + k] * w[k];
             }
-            for (; r < rank; ++r) value += latent_lds[r] * (float)u[(size_t)r * v];
-        } else {
-            value = (float)y[((size_t)head * n_tokens + t) * v + j];
+            for (; r < r1; ++r) value += (float)row[r] * (float)u[(size_t)r * v];
         }
-        out[((size_t)t * heads + head) * v + j] = (T)(value * g);
+        partial[wave][lane] = value;
+        __syncthreads();
+        if (wave) return;
+        value = 0.f;
+        for (int w = 0; w < waves; ++w) value += partial[w][lane];
+    } else {                            // nothing to multiply: one workgroup gates the head's whole row
+        float g = 1.f;
+        if (gate_column >= 0) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + head]));
+        for (int i = threadIdx.x; i < v; i += blockDim.x)
+            out[((size_t)t * heads + head) * v + i] = (T)((float)y[((size_t)head * n_tokens + t) * v + i] * g);
+        return;
     }
+    if (j >= v) return;
+    float g = 1.f;
+    if (gate_column >= 0) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + head]));
+    out[((size_t)t * heads + head) * v + j] = (T)(value * g);
 }
 
 LSA_EXPORT int lsa_latent_prepare(int code, const void* proj, long proj_stride, const void* q_latent, const void* up_keys,
@@ -131,10 +147,9 @@ LSA_EXPORT int lsa_latent_prepare(int code, const void* proj, long proj_stride, 
                                   int rank, int row_width, int write_cache, int n_tokens, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (rank + rot_dim > row_width || 2 * pairs > rot_dim || page_size <= 0 || (q_latent == nullptr) == (up_keys == nullptr)) return -1;
-    const size_t lds = up_keys ? (size_t)dim * sizeof(float) : 0;
-    if (lds > 60000) return -1;
-    dim3 grid(n_tokens, heads + 1);
-#define LSA_LAUNCH(T) latent_prepare_kernel<T><<<grid, 256, lds, stream>>>((const T*)proj, proj_stride, (const T*)q_latent, (const T*)up_keys, \
+    // (256 threads where the product is made here and for the cache row's norm; the copy alone needs a wavefront a piece)
+    dim3 grid(n_tokens, heads + 1, up_keys ? (row_width + 63) / 64 : 1);
+#define LSA_LAUNCH(T) latent_prepare_kernel<T><<<grid, 256, 0, stream>>>((const T*)proj, proj_stride, (const T*)q_latent, (const T*)up_keys, \
         norm_weight, eps, cos_sin, pairs, (T*)keys, (T*)values, table, table_stride, token_row, positions, page_size, (T*)out_q, heads, dim, \
         rot_dim, rank, row_width, write_cache, n_tokens)
     if (code) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
@@ -146,10 +161,8 @@ LSA_EXPORT int lsa_gate_heads(int code, const void* y, const void* mixed, const 
                               long proj_stride, int gate_column, void* out, int heads, int v, int n_tokens, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if ((y == nullptr) == (up_values == nullptr) || (up_values != nullptr && (mixed == nullptr || rank > row_width))) return -1;
-    const size_t lds = up_values ? (size_t)rank * sizeof(float) : 0;
-    if (lds > 60000) return -1;
-    dim3 grid(n_tokens, heads);
-#define LSA_LAUNCH(T) gate_heads_kernel<T><<<grid, 256, lds, stream>>>((const T*)y, (const T*)mixed, (const T*)up_values, rank, row_width, \
+    dim3 grid(n_tokens, heads, up_values ? (v + 63) / 64 : 1);
+#define LSA_LAUNCH(T) gate_heads_kernel<T><<<grid, up_values ? 256 : 64, 0, stream>>>((const T*)y, (const T*)mixed, (const T*)up_values, rank, row_width, \
         (const T*)proj, proj_stride, gate_column, (T*)out, heads, v, n_tokens)
     if (code) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
 #undef LSA_LAUNCH
