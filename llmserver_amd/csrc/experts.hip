@@ -303,13 +303,19 @@ __global__ __launch_bounds__(256) void experts_tile_kernel(const bf16_t* __restr
     constexpr int BN = 32 * NT;                                    // rows of B a block takes
     __shared__ __align__(16) bf16_t b_lds[BN * ROW];
     __shared__ int rows_of[TILE_M];
-    const int expert = tile_expert[blockIdx.x];
+    // Workgroups go to the eight XCDs in turn by their number.  The tiles of one expert stand next to each other in the
+    // list; numbered so that neighbours in the list get numbers eight apart, they run on one XCD at about the same time
+    // and the expert's rows are fetched into one L2 instead of several.
+    const int total = gridDim.x * gridDim.y, number = blockIdx.y * gridDim.x + blockIdx.x, share = total / 8;
+    const int place = number < share * 8 ? (number % 8) * share + number / 8 : number;
+    const int tile = place % gridDim.x, block_n = place / gridDim.x;
+    const int expert = tile_expert[tile];
     if (expert < 0) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, quad = lane >> 4;
     const int wave_m = wave >> 1, wave_n = wave & 1;
-    if (threadIdx.x < TILE_M) rows_of[threadIdx.x] = sorted[blockIdx.x * TILE_M + threadIdx.x];
+    if (threadIdx.x < TILE_M) rows_of[threadIdx.x] = sorted[tile * TILE_M + threadIdx.x];
     __syncthreads();
-    const int n0 = blockIdx.y * (GATED ? BN / 2 : BN);             // first output column of the block
+    const int n0 = block_n * (GATED ? BN / 2 : BN);                // first output column of the block
     const bf16_t* bm = b + (size_t)expert * expert_stride;
     // which rows of B the block's LDS rows are: GATED: the first half gate rows n0 + r, the second half their up rows
     auto b_row = [&](int r) {
