@@ -1,7 +1,7 @@
 from .attention import AttentionNames, AttentionPlan, AttentionTuning, GQAttention, TileLaunchCost, build_attention_plan, group_tiling
 from .base import (INT_TABLE, MATRIX, VECTOR, Block, FeedForward, Mixer, Norm, PagedAndStateSpec, PagedKVSpec, ParamSpec, Part,
                    PositionEncoding, StateSpec)
-from .block import DepthAverage, PostNormBlock, PreNormBlock
+from .block import DepthAverage, PostNormBlock, PreNormBlock, SandwichBlock
 from .conv import ShortConvolution
 from .embedding import NormedTokenEmbedding, TokenEmbedding
 from .experts import RoutedExperts
@@ -10,10 +10,13 @@ from .latent_attention import LatentAttention, LatentAttentionNames
 from .linear import Linear
 from .mlp import GatedMLP, GatedMLPNames
 from .norm import RMSNorm
+from .parallel import ParallelMixers, ScaledPair
+from .recurrent import GatedLinearAttention, GatedLinearAttentionNames, TimeMixing, TimeMixingNames, TokenShift
 from .rope import NoPosition, PairedRotaryPosition, RotaryPosition
 
 __all__ = ["KernelNamespace", "AttentionNames", "AttentionTuning", "TileLaunchCost", "GatedMLPNames", "AttentionPlan", "GQAttention", "build_attention_plan", "group_tiling", "INT_TABLE", "MATRIX", "VECTOR",
            "Block", "FeedForward", "Mixer", "Norm", "PagedKVSpec", "ParamSpec", "Part", "PositionEncoding",
            "StateSpec", "PreNormBlock", "TokenEmbedding", "Linear", "GatedMLP", "RMSNorm", "NoPosition",
            "RotaryPosition", "PairedRotaryPosition", "PagedAndStateSpec", "DepthAverage", "PostNormBlock", "ShortConvolution",
-           "NormedTokenEmbedding", "RoutedExperts", "LatentAttention", "LatentAttentionNames"]
+           "NormedTokenEmbedding", "RoutedExperts", "LatentAttention", "LatentAttentionNames", "SandwichBlock", "ParallelMixers",
+           "ScaledPair", "GatedLinearAttention", "GatedLinearAttentionNames", "TimeMixing", "TimeMixingNames", "TokenShift"]

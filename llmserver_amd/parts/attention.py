@@ -449,45 +449,68 @@ class GQAttention(Mixer):
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
                  window: Optional[int] = None, scale: Optional[float] = None, names: AttentionNames = AttentionNames(),
-                 sinks: Optional[str] = None):
+                 sinks: Optional[str] = None, softcap: Optional[float] = None, value_dim: Optional[int] = None,
+                 bare_names: bool = False):
         """``sinks``: the checkpoint name of a float vector ``[n_heads]`` whose exponentials join the softmax's
-        denominators (one term per head, without a key or a value), or None."""
+        denominators (one term per head, without a key or a value), or None.  ``softcap``: scores become
+        ``softcap * tanh(score / softcap)`` (after the scale, before the mask), or None.  ``value_dim``: the size of a
+        head's values if it is not the size of its queries and keys.  ``bare_names``: the names are the tensors' whole
+        names (no ``.weight`` behind them).
+
+        A position encoding that turns neighbouring dimensions together (``pairing == "neighbours"``), a rotation of a
+        part of the head, values of another size than the keys, and head sizes that are no multiple of 16 go the general
+        way: a kernel of its own normalises and rotates, and writes the cache rows and the query rows filled up with
+        zeros to the next head size the attention kernels take."""
         if n_heads % n_kv_heads:
             raise ValueError(f"Number of query heads must be divisible by the number of KV heads: query heads: {n_heads}, KV heads: {n_kv_heads}")
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.value_dim = head_dim if value_dim is None else int(value_dim)
         self.group_size = n_heads // n_kv_heads
-        if position.rotary_dim is not None and position.rotary_dim != head_dim:
-            raise ValueError(f"the position encoding rotates {position.rotary_dim} of a head's {head_dim} dimensions; this mixer's "
-                             "kernels rotate the whole head or nothing (a rotation of a part of the head is not built)")
+        paired = getattr(position, "pairing", None) == "neighbours"
+        self.general = paired or self.value_dim != head_dim or head_dim % 16 != 0 or \
+            (position.rotary_dim is not None and position.rotary_dim != head_dim)
+        if self.general:
+            if position.rotary_dim is not None and (not paired or position.rotary_dim > head_dim):
+                raise ValueError(f"the position encoding rotates {position.rotary_dim} of a head's {head_dim} dimensions; a rotation of a "
+                                 "part of the head is built for encodings that turn neighbouring dimensions together")
+            if bias:
+                raise ValueError("the general way of preparing queries, keys and values takes projections without biases")
+        self.row = -(-max(head_dim, self.value_dim) // 16) * 16      # a head as the attention kernels and the pages see it
         self.position = position
         self.qk_norm_eps = qk_norm_eps
         self.window = window
+        self.softcap = float(softcap) if softcap else None
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
-        q_rows, kv_rows = n_heads * head_dim, n_kv_heads * head_dim
-        stacked = {3: (q_rows, kv_rows, kv_rows), 2: (q_rows, 2 * kv_rows), 1: (q_rows + 2 * kv_rows,)}
+        q_rows, k_rows, v_rows = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * self.value_dim
+        stacked = {3: (q_rows, k_rows, v_rows), 2: (q_rows, k_rows + v_rows), 1: (q_rows + k_rows + v_rows,)}
         if len(names.qkv) not in stacked:
             raise ValueError(f"queries, keys and values come in one, two or three checkpoint tensors, not {len(names.qkv)}")
-        self.names = names
-        self.qkv = Linear(width, names.qkv, stacked[len(names.qkv)], bias)
-        self.o = Linear(q_rows, (names.out,), (width,), bias if out_bias is None else out_bias)
+        self.names, self.bare_names = names, bare_names
+        self.qkv = Linear(width, names.qkv, stacked[len(names.qkv)], bias, bare_names=bare_names)
+        self.o = Linear(n_heads * self.value_dim, (names.out,), (width,), bias if out_bias is None else out_bias, bare_names=bare_names)
         self.q_norm_weight = None
         self.k_norm_weight = None
         self.sinks_name, self.sinks = sinks, None
+        self._o_padded = None
 
     def cache_spec(self):
-        return PagedKVSpec(self.n_kv_heads, self.head_dim, self.window)
+        return PagedKVSpec(self.n_kv_heads, self.row, self.window)
+
+    def _norm_names(self):
+        suffix = "" if self.bare_names else ".weight"
+        return self.names.q_norm + suffix, self.names.k_norm + suffix
 
     def param_specs(self):
         specs = {**self.qkv.param_specs(), **self.o.param_specs()}
         if self.qk_norm_eps is not None:
-            specs[f"{self.names.q_norm}.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
-            specs[f"{self.names.k_norm}.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
+            for name in self._norm_names():
+                specs[name] = ParamSpec((self.head_dim,), VECTOR, "norm")
         if self.sinks_name is not None:
             specs[self.sinks_name] = ParamSpec((self.n_heads,), VECTOR, "normal")
         return specs
 
     def assign(self, name, tensor):
-        owner = name.rsplit(".", 1)[0]
+        owner = name if self.bare_names else name.rsplit(".", 1)[0]
         if name == self.sinks_name:
             self.sinks = tensor
         elif owner == self.names.q_norm:
@@ -504,9 +527,16 @@ class GQAttention(Mixer):
     def finalize(self):
         self.qkv.finalize()
         self.o.finalize()
+        if self.row != self.value_dim:
+            # The attention kernels leave a head's result in a row of `row` numbers, zeros behind the values: the output
+            # projection reads those rows as they are, through columns of zeros.
+            weight = self.o.weight
+            padded = weight.new_zeros((weight.shape[0], self.n_heads, self.row))
+            padded[:, :, :self.value_dim] = weight.view(weight.shape[0], self.n_heads, self.value_dim)
+            self._o_padded = padded.view(weight.shape[0], self.n_heads * self.row).contiguous()
 
     def plan_key(self):
-        return ("paged_attention", self.group_size, self.n_kv_heads, self.window, self.head_dim)
+        return ("paged_attention", self.group_size, self.n_kv_heads, self.window, self.row)
 
     def graph_shape(self, rows: int, longest_context: int):
         return "short contexts" if longest_context <= SHORT_CONTEXT else None
@@ -521,12 +551,36 @@ class GQAttention(Mixer):
             pairs = new_tokens * first + new_tokens * (new_tokens + 1) // 2
         else:
             pairs = sum(min(position + 1, self.window) for position in range(first, context))
-        return 4.0 * self.n_heads * self.head_dim * pairs
+        return 2.0 * self.n_heads * (self.head_dim + self.value_dim) * pairs
 
     def prepare(self, ctx):
-        stage_attention_plan(ctx, self.plan_key(), self.group_size, self.n_kv_heads, self.head_dim, self.window, self.graph_shape)
+        stage_attention_plan(ctx, self.plan_key(), self.group_size, self.n_kv_heads, self.row, self.window, self.graph_shape)
+
+    def _forward_general(self, x, ctx, cache, sink):
+        """Norm, rotation of neighbouring pairs, rows filled up to the kernels' head size: a kernel in front of attention."""
+        qkv = self.qkv.forward(x, ctx)
+        table = ctx.block_table(cache.group)
+        n = qkv.shape[0]
+        q = ctx.empty((n, self.n_heads * self.row))
+        ctx.ops.qkv_prepare(qkv, cache.keys, cache.values, table, ctx.token_row, ctx.positions, self.q_norm_weight, self.k_norm_weight,
+                            self.qk_norm_eps if self.qk_norm_eps is not None else 0.0, self.position.cos_sin(ctx), cache.page_size,
+                            self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, q, cache.writable)
+        out = ctx.empty((n, self.n_heads * self.row))
+        extra = {}
+        if self.sinks is not None:
+            extra["sinks"] = self.sinks
+        if self.softcap is not None:
+            extra["softcap"] = self.softcap
+        ctx.ops.paged_attention(q, out, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
+                                ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size,
+                                self.n_heads, self.n_kv_heads, self.row, ctx, **extra)
+        if self._o_padded is None:
+            return self.o.forward(out, ctx, sink=sink)
+        return ctx.ops.linear(out, self._o_padded)
 
     def forward(self, x, ctx, cache, sink=None):
+        if self.general:
+            return self._forward_general(x, ctx, cache, sink)
         qkv = self.qkv.forward(x, ctx)
         table = ctx.block_table(cache.group)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
@@ -546,6 +600,8 @@ class GQAttention(Mixer):
         extra = {"decode_fusion": fusion} if fusion is not None else {}
         if self.sinks is not None:
             extra["sinks"] = self.sinks
+        if self.softcap is not None:
+            extra["softcap"] = self.softcap
         ctx.ops.paged_attention(
             qkv, out, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
             ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size,

@@ -30,6 +30,14 @@ class ParamSpec:
     # The share of the tensor that one token's pass uses: 1 for a dense layer's matrix, k/n for one of n experts of
     # which a token chooses k, 0 for a table of which a token reads a row.  (What a step costs is summed from this.)
     share_per_token: float = 1.0
+    # Dimensions whose size the checkpoint decides (an inner rank that no configuration key names): ``shape`` holds
+    # what random weights draw there, a loader accepts any size, and the part reads the size off the tensor it is given.
+    free_dims: Tuple[int, ...] = ()
+
+    def fits(self, shape) -> bool:
+        """Whether a checkpoint tensor of ``shape`` can be this tensor."""
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(a == b or i in self.free_dims for i, (a, b) in enumerate(zip(shape, self.shape)))
 
 
 @dataclasses.dataclass(frozen=True)

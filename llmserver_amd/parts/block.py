@@ -181,3 +181,83 @@ class PostNormBlock(Block):
         result = ctx.empty(x.shape, dtype=torch.float32)
         ops.scaled_norm_add(out, fed, self.ffn_norm.weight, self.scale2, self.ffn_norm.eps, result, **after)
         return result, None
+
+
+class SandwichBlock(Block):
+    """A norm in front of every sublayer and one behind it: ``x <- x + n1b(mixer(n1(x)))``, then
+    ``x <- x + n2b(ffn(n2(x)))``, the stream in 32-bit throughout; ``ffn`` may be None.  The norm behind a sublayer, the
+    sum with the stream and the norm in front of the next sublayer are one kernel (``ops.norm_add_norm``); a mixer that
+    returns two results with scales (:class:`~llmserver_amd.parts.parallel.ScaledPair`) has them added up there too."""
+    takes_following = True
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, mixer_out_norm: Norm, ffn_norm=None, ffn=None, ffn_out_norm=None,
+                 names=("norm1", "mix", "norm1b", "norm2", "mlp", "norm2b")):
+        self.mixer_norm, self.mixer, self.mixer_out_norm = mixer_norm, mixer, mixer_out_norm
+        self.ffn_norm, self.ffn, self.ffn_out_norm = ffn_norm, ffn, ffn_out_norm
+        self.names = tuple(names)
+
+    def _parts(self):
+        parts = dict(zip(self.names[:3], (self.mixer_norm, self.mixer, self.mixer_out_norm)))
+        if self.ffn is not None:
+            parts.update(zip(self.names[3:], (self.ffn_norm, self.ffn, self.ffn_out_norm)))
+        return parts
+
+    def param_specs(self):
+        return {f"{prefix}.{name}" if name else prefix: spec for prefix, part in self._parts().items()
+                for name, spec in part.param_specs().items()}
+
+    def assign(self, name, tensor):
+        parts = self._parts()
+        if name in parts:                                   # the part's name is the tensor's
+            parts[name].assign("", tensor)
+            return
+        prefix, rest = name.split(".", 1)
+        parts[prefix].assign(rest, tensor)
+
+    def finalize(self):
+        for part in self._parts().values():
+            part.finalize()
+
+    def entry_norm(self):
+        return self.mixer_norm
+
+    @staticmethod
+    def _update(ctx, x, result, norm, following):
+        """``x + norm(result)`` and, if ``following`` is given, that norm of the sum in the compute type."""
+        from .parallel import ScaledPair
+        second, scales = None, None
+        if isinstance(result, ScaledPair):
+            result, second, scales = result.left, result.right, (result.left_scale, result.right_scale)
+        out = ctx.empty(x.shape, dtype=torch.float32)
+        normed = ctx.empty(x.shape) if following is not None else None
+        ctx.ops.norm_add_norm(x, result, norm.weight, norm.eps, out, following.weight if following is not None else None,
+                              following.eps if following is not None else 0.0, normed, second, scales)
+        return out, normed
+
+    def forward(self, resid, delta, ctx, cache, following=None):
+        """``delta``: None, or a :class:`StreamUpdate` whose ``normed`` rows are the stream under this block's first norm
+        (the block before was told that norm as its ``following`` and has carried it out)."""
+        x, h = resid, None
+        if isinstance(delta, StreamUpdate):
+            x = delta.resid
+            h = delta.normed if delta.norm is self.mixer_norm else None
+        elif delta is not None:
+            raise ValueError("this block takes a stream to which everything has been added")
+        if h is None:
+            h = ctx.empty(x.shape)
+            ctx.ops.norm_rows(x, None, self.mixer_norm.weight, self.mixer_norm.eps, h)
+        mixed = self.mixer.forward(h, ctx, cache)
+        if self.ffn is None:
+            return self._handed_on(*self._update(ctx, x, mixed, self.mixer_out_norm, self._same_kind(following)), following)
+        x, h = self._update(ctx, x, mixed, self.mixer_out_norm, self.ffn_norm)
+        fed = self.ffn.forward(h, ctx)
+        return self._handed_on(*self._update(ctx, x, fed, self.ffn_out_norm, self._same_kind(following)), following)
+
+    @staticmethod
+    def _handed_on(x, normed, following):
+        return x, (StreamUpdate(following, x, normed=normed) if normed is not None else None)
+
+    @staticmethod
+    def _same_kind(following):
+        """The next block's first norm, if its kernel can be folded in here (a plain RMS norm of the stream)."""
+        return following if following is not None and hasattr(following, "weight") and hasattr(following, "eps") else None

@@ -7,18 +7,25 @@ from .base import MATRIX, ParamSpec, Part
 
 
 class TokenEmbedding(Part):
-    def __init__(self, vocab: int, width: int):
-        self.vocab, self.width = vocab, width
+    """``tensor``: the table's name below the part's own ("" if the part's name is the tensor's).  ``wide``: the rows
+    start a residual stream that is kept in 32-bit whatever the type of the table."""
+
+    def __init__(self, vocab: int, width: int, tensor: str = "weight", wide: bool = False):
+        self.vocab, self.width, self.tensor, self.wide = vocab, width, tensor, wide
         self.weight = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.vocab, self.width), MATRIX, "normal", share_per_token=0.0)}
+        return {self.tensor: ParamSpec((self.vocab, self.width), MATRIX, "normal", share_per_token=0.0)}
 
     def assign(self, name, tensor):
-        assert name == "weight"
+        assert name == self.tensor
         self.weight = tensor
 
     def forward(self, token_ids, ctx):
+        if self.wide:
+            out = ctx.empty((token_ids.shape[0], self.width), dtype=torch.float32)
+            ctx.ops.embedding_wide(self.weight, token_ids, out)
+            return out
         out = ctx.empty((token_ids.shape[0], self.width))
         ctx.ops.embedding(self.weight, token_ids, out)
         return out

@@ -1,7 +1,11 @@
 """Routed experts: every token's feed-forward is a weighted sum of ``top`` of ``experts`` small gated feed-forwards.
 
-Router logits ``z = R h`` in 32-bit; the ``top`` largest are chosen (the first of equal ones) and weighted by the softmax
-over the chosen logits only.  Expert: ``D (act(G h) * (U h))`` with ``act = silu``; no biases.  The experts' matrices
+Router logits ``z = R h`` in 32-bit.  ``scoring="softmax"``: the ``top`` largest logits are chosen (the first of equal
+ones) and weighted by the softmax over the chosen logits only.  ``scoring="sigmoid"``: scores ``sigmoid(z)``; with
+``groups=(count, keep)`` the experts form ``count`` equal groups of neighbours, a group's score is the sum of its two
+largest scores, and only experts of the ``keep`` best groups can be chosen; the ``top`` largest scores are chosen and
+are the weights as they are.  Expert: ``D (act(G h) * (U h))`` with ``act = silu``, or, with ``activation="clamped"``,
+``g = min(G h, limit)``, ``u = clamp(U h, -limit, limit)``, ``D (g * sigmoid(1.702 g) * (u + 1))``; no biases.  The experts' matrices
 are stacked (``[experts, 2F, W]`` gate rows then up rows, ``[experts, W, F]``), and the kernels pick each token's from
 the list of chosen experts on the device: nothing of the routing is read on the host.
 """
@@ -15,10 +19,24 @@ from .base import VECTOR, FeedForward, ParamSpec
 class RoutedExperts(FeedForward):
     reads_stream = True       # forward takes ``stream=``: the 32-bit rows that ``x`` was rounded from, for the router
 
+    SCORINGS = ("softmax", "sigmoid")
+    ACTIVATIONS = ("silu", "clamped")
+
     def __init__(self, width: int, intermediate: int, experts: int, top: int, router: str = "router", expert: str = "e{}",
-                 pieces=("gate", "up", "down")):
+                 pieces=("gate", "up", "down"), scoring: str = "softmax", groups=None, activation: str = "silu", limit: float = 0.0,
+                 reads_stream: bool = True):
         if not 1 <= top <= experts:
             raise ValueError(f"a token uses {top} of {experts} experts")
+        if scoring not in self.SCORINGS or activation not in self.ACTIVATIONS:
+            raise ValueError(f"scoring {scoring!r} / activation {activation!r}: built are {self.SCORINGS} and {self.ACTIVATIONS}")
+        if groups is not None:
+            count, keep = groups
+            if scoring != "sigmoid" or experts % count or not 1 <= keep <= count or top > keep * (experts // count):
+                raise ValueError(f"{experts} experts in {count} groups of which {keep} are kept, {top} chosen, scoring {scoring!r}")
+        if activation == "clamped" and not limit > 0.0:
+            raise ValueError("the clamped activation needs its limit")
+        self.scoring, self.groups, self.activation, self.limit = scoring, tuple(groups) if groups is not None else None, activation, float(limit)
+        self.reads_stream = reads_stream
         self.width, self.intermediate, self.experts, self.top = width, intermediate, experts, top
         self.router_name, self.expert_name, self.pieces = router, expert, tuple(pieces)
         self._parts = {}
@@ -60,11 +78,13 @@ class RoutedExperts(FeedForward):
         n = x.shape[0]
         chosen = ctx.empty((n, self.top), dtype=torch.int32)
         weights = ctx.empty((n, self.top), dtype=torch.float32)
-        ops.route_experts(x if stream is None else stream, self.router, self.top, chosen, weights)
+        extra = {} if self.scoring == "softmax" else {"scoring": self.scoring, "groups": self.groups}
+        ops.route_experts(x if stream is None else stream, self.router, self.top, chosen, weights, **extra)
         out = ctx.empty((n, self.width), dtype=torch.float32)
-        if ops.experts_sorted(x, self.gate_up, self.down, chosen, weights, out):       # many tokens: pairs sorted by expert
+        extra = {} if self.activation == "silu" else {"activation": self.activation, "limit": self.limit}
+        if ops.experts_sorted(x, self.gate_up, self.down, chosen, weights, out, **extra):       # many tokens: pairs sorted by expert
             return out
         hidden = ctx.empty((n * self.top, self.intermediate))
-        ops.experts_gate_up(x, self.gate_up, chosen, hidden)
+        ops.experts_gate_up(x, self.gate_up, chosen, hidden, **extra)
         ops.experts_down(hidden, self.down, chosen, weights, out)
         return out

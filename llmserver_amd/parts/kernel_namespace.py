@@ -45,14 +45,73 @@ class KernelNamespace:
         raise NotImplementedError
 
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None, softcap=None):
         """``sinks [n_q]`` (float32) or None: one more term ``exp(sinks[head])`` in every softmax's denominator, with no
-        key and no value.  ``qkv`` may hold the queries only (``[T, n_q * head_dim]``) where nothing is fused."""
+        key and no value.  ``softcap`` (a number or None): scaled scores become ``softcap * tanh(score / softcap)`` before
+        the mask.  ``qkv`` may hold the queries only (``[T, n_q * head_dim]``) where nothing is fused."""
+        raise NotImplementedError
+
+    def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True):
+        """``qkv [T, n_q * dim + n_kv * dim + n_kv * value_dim]``.  Per head, queries and keys are RMS-normed over ``dim``
+        (``q_weight`` / ``k_weight [dim]`` float32, or both None: no norm), then the first ``2 * pairs`` dimensions turn
+        in neighbouring pairs (2i, 2i+1) by ``cos_sin [T, 2 * pairs]`` (cosines, then sines; None: no rotation).  With
+        ``D`` the pages' head size: ``out_q [T, n_q * D]`` gets the query rows, zeros behind ``dim``; with ``write_cache``,
+        ``keys [pages, n_kv, page_size, D]`` get the key rows and ``values [pages, n_kv, D, page_size]`` the value rows
+        (zeros behind ``dim`` / ``value_dim``) at every token's place."""
+        raise NotImplementedError
+
+    # Recurrent mixers.
+    def token_shift(self, h, mu, state, offset, state_slots, token_row, positions, row_start, out, keep=False):
+        """``out[m, t] = h[t] + (before[t] - h[t]) * mu[m]``, ``mu [M, W]`` float32, ``out [M, T, W]`` of ``h``'s type.
+        ``before[t]``: the row of the token before ``t`` in its request: a row of this step, or, for a row's first
+        token, ``state[slot, offset : offset + W]`` (float32; zeros at position 0 whatever the state holds).  ``keep``
+        (steps of one token per row only): the state also becomes this step's row, as :meth:`token_shift_keep` would do."""
+        raise NotImplementedError
+
+    def token_shift_keep(self, h, state, offset, state_slots, row_start, row_len):
+        """``state[slot, offset : offset + W] =`` every row's last row of ``h`` (rows without tokens keep theirs)."""
+        raise NotImplementedError
+
+    def batched_linear(self, x, weights):
+        """``x [B, T, in]``, ``weights [B, out, in]`` -> ``[B, T, out]`` of ``x``'s type, 32-bit sums."""
+        raise NotImplementedError
+
+    def tanh_(self, x):
+        raise NotImplementedError
+
+    def linear_recurrence(self, q, k, v, decay, decay_bias, decay_mode, tau, bonus, q_scale, state, offset, state_slots,
+                          row_start, row_len, row_ctx, out, heads, dim, value_dim):
+        """Per row (request) and head, over the row's tokens in order: ``d_t = decay(decay[t] + decay_bias)`` per key
+        channel (``"sigmoid_root"``: ``sigmoid(z)^(1/tau)``; ``"double_exp"``: ``exp(-exp(z))``), all float32.  ``bonus``
+        None: ``S = diag(d_t) S + k_t v_t^T``, ``out_t = S^T (q_t * q_scale)``.  ``bonus [heads, dim]``:
+        ``out_t = (S + diag(bonus) k_t v_t^T)^T (q_t * q_scale)``, then ``S = diag(d_t) S + k_t v_t^T``.
+        ``q, k [T, heads * dim]``, ``v [T, heads * value_dim]`` (views with unit stride along a row), ``decay [T, heads *
+        dim]`` float32, ``out [T, heads * value_dim]`` float32.  ``S [heads, dim, value_dim]`` float32 lies in
+        ``state[slot, offset:]``; a row whose first token stands at position 0 starts from zeros whatever the slot holds;
+        the state after the row's last token is stored back."""
+        raise NotImplementedError
+
+    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim):
+        """``out[t, h, :] = x[t, h, :] / rms(x[t, h, :]) * w * silu(gate[t, h, :])``; ``x`` float32, ``w = weight [value_dim]``
+        shared by the heads or, with ``weight_per_channel``, ``weight [heads * value_dim]``; ``gate`` a view like ``out``."""
+        raise NotImplementedError
+
+    def scaled_sum(self, x, x_scale, y, y_scale, out):
         raise NotImplementedError
 
     # A residual stream kept in 32-bit beside activations of the compute type.
     def embedding_norm(self, table, token_ids, weight, eps, out):
         """``out [T, W]`` float32 ``= rmsnorm(table[token_ids]) * weight``."""
+        raise NotImplementedError
+
+    def embedding_wide(self, table, token_ids, out):
+        """``out [T, W]`` float32 ``= table[token_ids]``."""
+        raise NotImplementedError
+
+    def norm_add_norm(self, x, y, weight, eps, out, next_weight=None, next_eps=0.0, normed=None, y2=None, scales=None):
+        """``out = x + rmsnorm(y') * weight`` in float32, with ``y' = y`` or, with ``y2`` and ``scales = (a, b)``,
+        ``a * y + b * y2``; with ``next_weight``: ``normed = rmsnorm(out) * next_weight`` (eps ``next_eps``, any type)."""
         raise NotImplementedError
 
     def norm_rows(self, x, rows, weight, eps, out):
@@ -93,12 +152,16 @@ class KernelNamespace:
         raise NotImplementedError
 
     # Routed experts.
-    def route_experts(self, x, router, top, chosen, weights):
-        """Float32 logits ``x router^T``; ``chosen [T, top]`` the largest (first of equals), ``weights`` their softmax."""
+    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None):
+        """Float32 logits ``x router^T``; ``chosen [T, top]`` the largest (first of equals), ``weights`` their softmax.
+        ``scoring="sigmoid"``: scores ``sigmoid(logits)``, the largest scores chosen, the scores themselves the weights;
+        ``groups=(count, keep)``: only experts of the ``keep`` best of ``count`` equal groups of neighbours can be chosen,
+        a group's score the sum of its two largest scores (the first of equal groups)."""
         raise NotImplementedError
 
-    def experts_gate_up(self, x, gate_up, chosen, hidden):
-        """``hidden[t * top + s] = silu(G x_t) * (U x_t)`` with ``[G; U] = gate_up[chosen[t, s]]`` (``[E, 2F, W]``)."""
+    def experts_gate_up(self, x, gate_up, chosen, hidden, activation="silu", limit=0.0):
+        """``hidden[t * top + s] = silu(G x_t) * (U x_t)`` with ``[G; U] = gate_up[chosen[t, s]]`` (``[E, 2F, W]``);
+        ``activation="clamped"``: ``g = min(G x, limit)``, ``u = clamp(U x, -limit, limit)``, ``g * sigmoid(1.702 g) * (u + 1)``."""
         raise NotImplementedError
 
     def experts_down(self, hidden, down, chosen, weights, out):
@@ -114,7 +177,7 @@ class KernelNamespace:
         products themselves (``up_keys=`` / ``up_values=``) instead of getting them from batched products made before."""
         return False
 
-    def experts_sorted(self, x, gate_up, down, chosen, weights, out) -> bool:
+    def experts_sorted(self, x, gate_up, down, chosen, weights, out, activation="silu", limit=0.0) -> bool:
         """Both products of the routed experts and the weighted sum for all of the step's tokens at once, the (token,
         expert) pairs sorted by expert so that an expert's matrices are read once per tile of pairs: ``out`` as
         :meth:`experts_down` leaves it.  False: not done (not offered, or it would not pay for these sizes)."""

@@ -1,4 +1,4 @@
-"""Gated feed-forward ``down(act(gate(x)) * up(x))``; ``act`` is SiLU in every model built so far.
+"""Gated feed-forward ``down(act(gate(x)) * up(x))``; ``act`` is SiLU or the tanh form of GELU.
 
 Gate and up are one stacked product, gate first (utils/layers.py:194-218;
 utils/fused_ops.py:59-61, 80-88).  Sigmoid and the product run in 32-bit inside
@@ -27,10 +27,11 @@ class GatedMLP(FeedForward):
 
     # config.json's names of an activation -> the name the kernels know it by (utils/layers.py:182 in the
     # reference lists more; a further one is an entry here and a branch in the activation kernel and the gated epilogues)
-    ACTIVATIONS = {"silu": "silu", "swish": "silu"}
+    ACTIVATIONS = {"silu": "silu", "swish": "silu", "gelu_tanh": "gelu_tanh", "gelu_pytorch_tanh": "gelu_tanh"}
 
     def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False,
-                 names: GatedMLPNames = GatedMLPNames()):
+                 names: GatedMLPNames = GatedMLPNames(), bare_names: bool = False):
+        """``bare_names``: the names are the tensors' whole names below the layer's (no ``.weight`` behind them)."""
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"Unsupported activation {activation!r}; supported: {sorted(self.ACTIVATIONS)}")
         self.activation = self.ACTIVATIONS[activation]
@@ -39,14 +40,16 @@ class GatedMLP(FeedForward):
         if len(names.gate_up) not in (1, 2):
             raise ValueError(f"gate and up projection come in one or two checkpoint tensors, not {len(names.gate_up)}")
         self.names = names
-        self.gate_up = Linear(width, names.gate_up, (intermediate, intermediate) if len(names.gate_up) == 2 else (2 * intermediate,), bias)
-        self.down = Linear(intermediate, (names.down,), (width,), bias)
+        self.bare_names = bare_names
+        self.gate_up = Linear(width, names.gate_up, (intermediate, intermediate) if len(names.gate_up) == 2 else (2 * intermediate,), bias,
+                              bare_names=bare_names)
+        self.down = Linear(intermediate, (names.down,), (width,), bias, bare_names=bare_names)
 
     def param_specs(self):
         return {**self.gate_up.param_specs(), **self.down.param_specs()}
 
     def assign(self, name, tensor):
-        owner = name.rsplit(".", 1)[0]
+        owner = name if self.bare_names else name.rsplit(".", 1)[0]
         if owner == self.names.down:
             self.down.assign(name, tensor)
         elif owner in self.names.gate_up:

@@ -53,7 +53,7 @@ def check_names(model, reader: CheckpointReader):
         if name in ignored:
             continue
         found = reader.shape(name)
-        if tuple(found) != tuple(specs[name].shape):
+        if not specs[name].fits(found):
             wrong.append((name, found, specs[name].shape))
     return missing, unexpected, wrong
 

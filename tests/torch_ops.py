@@ -65,7 +65,7 @@ class TorchOps(KernelNamespace):
         gate_up = self._scaled(x.float() @ gate_up_weight.float().t(), row_scale, x.shape[1])
         inter = gate_up.shape[1] // 2
         gate, up = gate_up[:, :inter], gate_up[:, inter:]
-        return (gate * torch.sigmoid(gate) * up).to(x.dtype)
+        return (self._activated(gate, activation) * up).to(x.dtype)
 
     def linear_partial_sums(self, x, weight, few_rows_too=False):
         if not self.fused or not (0 if few_rows_too else 16) < x.shape[0] <= 128:
@@ -105,10 +105,18 @@ class TorchOps(KernelNamespace):
         normed = total * torch.rsqrt(total.pow(2).mean(dim=-1, keepdim=True) + eps) * weight
         out.copy_(normed.to(out.dtype))
 
+    @staticmethod
+    def _activated(gate, activation):
+        if activation == "silu":
+            return gate * torch.sigmoid(gate)
+        if activation == "gelu_tanh":
+            return 0.5 * gate * (1.0 + torch.tanh(0.7978845608028654 * (gate + 0.044715 * gate ** 3)))
+        raise ValueError(f"no twin for the activation {activation!r}")
+
     def swiglu(self, gate_up, out, activation="silu"):
         inter = out.shape[1]
         gate, up = gate_up[:, :inter].float(), gate_up[:, inter:].float()
-        out.copy_((gate * torch.sigmoid(gate) * up).to(out.dtype))
+        out.copy_((self._activated(gate, activation) * up).to(out.dtype))
 
     def add_bias_(self, y, bias):
         y.copy_((y.float() + bias).to(y.dtype))
@@ -140,7 +148,7 @@ class TorchOps(KernelNamespace):
         values[pages, :, :, slots] = heads[:, n_q + n_kv:].to(values.dtype)
 
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None, softcap=None):
         """Per request row: gather its keys/values through the block table, one softmax over all
         keys a query may see (no tiles, no splits).  ``decode_fusion``: the step's rows bring one token each and
         ``qkv`` is the raw projection, which is left as it is."""
@@ -168,6 +176,8 @@ class TorchOps(KernelNamespace):
             k = k.repeat_interleave(group, dim=1)
             v = v.repeat_interleave(group, dim=1)
             scores = torch.einsum("qhd,khd->hqk", q, k) * scale
+            if softcap:
+                scores = softcap * torch.tanh(scores / softcap)
             q_pos = torch.arange(ctx_len - length, ctx_len, device=qkv.device)
             hidden = place[None, :] > q_pos[:, None]
             if window:
@@ -189,6 +199,16 @@ class TorchOps(KernelNamespace):
 
     def embedding_norm(self, table, token_ids, weight, eps, out):
         out.copy_(self._rms(table[token_ids.long()].float(), eps) * weight)
+
+    def embedding_wide(self, table, token_ids, out):
+        out.copy_(table[token_ids.long()].float())
+
+    def norm_add_norm(self, x, y, weight, eps, out, next_weight=None, next_eps=0.0, normed=None, y2=None, scales=None):
+        update = y.float() if y2 is None else scales[0] * y.float() + scales[1] * y2.float()
+        total = x + self._rms(update, eps) * weight
+        out.copy_(total)
+        if next_weight is not None:
+            normed.copy_((self._rms(total, next_eps) * next_weight).to(normed.dtype))
 
     def norm_rows(self, x, rows, weight, eps, out):
         picked = x if rows is None else x[rows.long()]
@@ -241,6 +261,106 @@ class TorchOps(KernelNamespace):
         if rounded is not None:
             rounded.copy_(s.to(rounded.dtype))
 
+    # -- general preparation of queries, keys and values -------------------------------------------------
+    def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True):
+        n, width = qkv.shape[0], keys.shape[-1]
+        q = qkv[:, :n_q * dim].float().view(n, n_q, dim)
+        k = qkv[:, n_q * dim:(n_q + n_kv) * dim].float().view(n, n_kv, dim)
+        v = qkv[:, (n_q + n_kv) * dim:].float().view(n, n_kv, value_dim)
+        if q_weight is not None:
+            q, k = self._rms(q, eps) * q_weight, self._rms(k, eps) * k_weight
+        if cos_sin is not None:
+            pairs = cos_sin.shape[1] // 2
+            cos, sin = cos_sin[:, None, :pairs], cos_sin[:, None, pairs:]
+
+            def turned(x):
+                a, b = x[..., 0:2 * pairs:2], x[..., 1:2 * pairs:2]
+                return torch.cat([torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1).flatten(-2), x[..., 2 * pairs:]], dim=-1)
+            q, k = turned(q), turned(k)
+        full = torch.zeros((n, n_q, width), dtype=torch.float32, device=qkv.device)
+        full[..., :dim] = q
+        out_q.copy_(full.view(n, n_q * width).to(out_q.dtype))
+        if not write_cache:
+            return
+        pos = positions.long()
+        pages = table.long()[token_row.long(), pos // page_size]
+        slots = pos % page_size
+        key_rows = torch.zeros((n, n_kv, width), dtype=torch.float32, device=qkv.device)
+        key_rows[..., :dim] = k
+        value_rows = torch.zeros((n, n_kv, width), dtype=torch.float32, device=qkv.device)
+        value_rows[..., :value_dim] = v
+        keys[pages, :, slots, :] = key_rows.to(keys.dtype)
+        values[pages, :, :, slots] = value_rows.to(values.dtype)
+
+    # -- recurrent mixers --------------------------------------------------------------------------------
+    def token_shift(self, h, mu, state, offset, state_slots, token_row, positions, row_start, out, keep=False):
+        width = h.shape[1]
+        before = torch.zeros_like(h, dtype=torch.float32)
+        for t in range(h.shape[0]):
+            row = int(token_row[t])
+            if int(positions[t]) == 0:
+                continue
+            before[t] = h[t - 1].float() if t > int(row_start[row]) else state[int(state_slots[row]), offset:offset + width]
+        wide = h.float()
+        out.copy_((wide[None] + (before - wide)[None] * mu[:, None, :]).to(out.dtype))
+        if keep:
+            assert h.shape[0] == len(row_start)
+            for t in range(h.shape[0]):
+                state[int(state_slots[int(token_row[t])]), offset:offset + width] = h[t].float()
+
+    def token_shift_keep(self, h, state, offset, state_slots, row_start, row_len):
+        width = h.shape[1]
+        for row in range(len(row_len)):
+            if int(row_len[row]) > 0:
+                state[int(state_slots[row]), offset:offset + width] = h[int(row_start[row]) + int(row_len[row]) - 1].float()
+
+    def batched_linear(self, x, weights):
+        return torch.bmm(x.float(), weights.float().transpose(1, 2)).to(x.dtype)
+
+    def tanh_(self, x):
+        x.copy_(torch.tanh(x.float()).to(x.dtype))
+
+    def linear_recurrence(self, q, k, v, decay, decay_bias, decay_mode, tau, bonus, q_scale, state, offset, state_slots,
+                          row_start, row_len, row_ctx, out, heads, dim, value_dim):
+        z = decay.float() + (decay_bias if decay_bias is not None else 0.0)
+        if decay_mode == "sigmoid_root":
+            factor = torch.exp(torch.nn.functional.logsigmoid(z) / tau)
+        elif decay_mode == "double_exp":
+            factor = torch.exp(-torch.exp(z))
+        else:
+            raise ValueError(decay_mode)
+        size = heads * dim * value_dim
+        for row in range(len(row_len)):
+            start, count, end = int(row_start[row]), int(row_len[row]), int(row_ctx[row])
+            if count <= 0:
+                continue
+            slot = int(state_slots[row])
+            matrix = state[slot, offset:offset + size].view(heads, dim, value_dim).clone()
+            if end - count == 0:
+                matrix.zero_()
+            for t in range(start, start + count):
+                qt = q[t].float().view(heads, dim) * q_scale
+                kv = k[t].float().view(heads, dim)[:, :, None] * v[t].float().view(heads, value_dim)[:, None, :]
+                d = factor[t].view(heads, dim)[:, :, None]
+                if bonus is None:
+                    matrix = d * matrix + kv
+                    out[t] = torch.einsum("hdv,hd->hv", matrix, qt).reshape(-1)
+                else:
+                    out[t] = torch.einsum("hdv,hd->hv", matrix + bonus[:, :, None] * kv, qt).reshape(-1)
+                    matrix = d * matrix + kv
+            state[slot, offset:offset + size] = matrix.reshape(-1)
+
+    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim):
+        n = x.shape[0]
+        normed = self._rms(x.float().view(n, heads, value_dim), eps)
+        normed = normed * (weight.view(heads, value_dim) if weight_per_channel else weight)
+        g = gate.float().view(n, heads, value_dim)
+        out.copy_((normed * g * torch.sigmoid(g)).reshape(n, heads * value_dim).to(out.dtype))
+
+    def scaled_sum(self, x, x_scale, y, y_scale, out):
+        out.copy_((x_scale * x.float() + y_scale * y.float()).to(out.dtype))
+
     # -- attention over a shared latent ------------------------------------------------------------------
     inside = False          # True: the parts are told to let latent_prepare and gate_heads make the per-head products
 
@@ -288,18 +408,42 @@ class TorchOps(KernelNamespace):
         out.copy_((y.float().transpose(0, 1) * gate[..., None]).reshape(n, heads * v).to(out.dtype))
 
     # -- routed experts ----------------------------------------------------------------------------------
-    def route_experts(self, x, router, top, chosen, weights):
-        best = torch.topk(x.float() @ router.float().t(), top, dim=-1)
-        chosen.copy_(best.indices.to(chosen.dtype))
-        weights.copy_(torch.softmax(best.values, dim=-1))
+    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None):
+        logits = x.float() @ router.float().t()
+        if scoring == "softmax":
+            best = torch.topk(logits, top, dim=-1)
+            chosen.copy_(best.indices.to(chosen.dtype))
+            weights.copy_(torch.softmax(best.values, dim=-1))
+            return
+        scores = torch.sigmoid(logits)
+        allowed = scores
+        if groups is not None:
+            count, keep = groups
+            per = scores.shape[1] // count
+            grouped = scores.view(-1, count, per)
+            group_scores = torch.topk(grouped, min(2, per), dim=-1).values.sum(dim=-1)
+            kept = torch.zeros_like(group_scores, dtype=torch.bool)
+            for _ in range(keep):                               # the best groups, the first of equal ones
+                pick = group_scores.masked_fill(kept, float("-inf")).argmax(dim=-1, keepdim=True)
+                kept.scatter_(1, pick, True)
+            allowed = scores.masked_fill(~kept[:, :, None].expand(-1, -1, per).reshape(scores.shape), float("-inf"))
+        for k in range(top):                                    # the largest scores, the first of equal ones
+            pick = allowed.argmax(dim=-1, keepdim=True)
+            chosen[:, k] = pick[:, 0].to(chosen.dtype)
+            weights[:, k] = scores.gather(1, pick)[:, 0]
+            allowed = allowed.scatter(1, pick, float("-inf"))
 
-    def experts_gate_up(self, x, gate_up, chosen, hidden):
+    def experts_gate_up(self, x, gate_up, chosen, hidden, activation="silu", limit=0.0):
         top, inter = chosen.shape[1], hidden.shape[1]
         for t in range(x.shape[0]):
             for s in range(top):
                 both = gate_up[int(chosen[t, s])].float() @ x[t].float()
                 gate, up = both[:inter], both[inter:]
-                hidden[t * top + s] = (gate * torch.sigmoid(gate) * up).to(hidden.dtype)
+                if activation == "clamped":
+                    gate, up = gate.clamp(max=limit), up.clamp(min=-limit, max=limit)
+                    hidden[t * top + s] = (gate * torch.sigmoid(1.702 * gate) * (up + 1.0)).to(hidden.dtype)
+                else:
+                    hidden[t * top + s] = (gate * torch.sigmoid(gate) * up).to(hidden.dtype)
 
     def experts_down(self, hidden, down, chosen, weights, out):
         top = chosen.shape[1]
