@@ -49,7 +49,24 @@ struct Geometry {
     unsigned page_magic;      // ceil(2^32 / page_size): key / page_size == mulhi(key, page_magic) for key < 2^32 / page_size
     float scale;
     const float* sinks;       // [n_q] or null: exp(sinks[head]) joins every softmax's denominator (no key, no value)
+    float cap, cap_inverse;   // cap > 0: a scaled score s becomes cap * tanh(s / cap) before the mask
+    float scale_inverse;      // 1 / scale (0 for a scale of 0), for the kernel that keeps its scores unscaled
 };
+
+__device__ __forceinline__ float tanh_of(float x) {
+#if LSA_BF16
+    // 1 - 2 / (e^(2x) + 1): off by a few 1e-7, far below what bfloat16 keeps of a probability; saturates to +-1
+    const float e = __builtin_amdgcn_exp2f(x * 2.885390081777927f);
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+#else
+    return tanhf(x);
+#endif
+}
+
+// The score as the softmax sees it, from the scaled dot product.
+__device__ __forceinline__ float capped(float scaled, const Geometry& g) {
+    return g.cap > 0.f ? g.cap * tanh_of(scaled * g.cap_inverse) : scaled;
+}
 
 // What the accumulated output of a pair is multiplied by at the very end: one over the sum of its keys' weights
 // (`total`, taken under the maximum `top`, in natural units with the scale applied) and, where the head has a sink, of
@@ -411,7 +428,7 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
         dot += __shfl_xor(dot, 16, 64);
         dot += __shfl_xor(dot, 32, 64);
         if (pair_valid) {
-            run_max = dot * g.scale;
+            run_max = capped(dot * g.scale, g);
             run_sum = quad == 0 ? 1.f : 0.f;
 #pragma unroll
             for (int c = 0; c < ND; ++c)
@@ -449,7 +466,7 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
             for (int r = 0; r < 4; ++r) {
                 const int kpos = kt + 16 * t2 + 4 * quad + r;
                 const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
-                const float v = seen ? s4[r] * g.scale : NEG_INF;
+                const float v = seen ? capped(s4[r] * g.scale, g) : NEG_INF;
                 sv[4 * t2 + r] = v;
                 tile_max = fmaxf(tile_max, v);
             }
@@ -468,7 +485,7 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
             for (int r = 0; r < 4; ++r) {
                 const int kpos = kt + 4 * quad + r;
                 const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
-                const float v = seen ? s4[r] * g.scale : NEG_INF;
+                const float v = seen ? capped(s4[r] * g.scale, g) : NEG_INF;
                 sv[r] = v;
                 tile_max = fmaxf(tile_max, v);
             }
@@ -915,6 +932,7 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     float v = s4[u][r];
+                    if (g.cap > 0.f) v = capped(v * g.scale, g) * g.scale_inverse;       // (scores stay in units of 1 / scale here)
                     if (!FULL) {
                         const int kpos = kt + 8 * quad + 4 * t2 + r;
                         const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos[u] && (g.window <= 0 || kpos > q_pos[u] - g.window);
@@ -1231,7 +1249,7 @@ __global__ __launch_bounds__(256) void paged_attention_tile_kernel_f32(
         for (int r = 0; r < 4; ++r) {
             const int kpos = kt + 4 * quad + r;
             const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
-            sv[r] = seen ? s4[r] * g.scale : NEG_INF;
+            sv[r] = seen ? capped(s4[r] * g.scale, g) : NEG_INF;
             step_max = fmaxf(step_max, sv[r]);
         }
         step_max = fmaxf(step_max, __shfl_xor(step_max, 16, 64));
@@ -1405,8 +1423,9 @@ LSA_EXPORT int lsa_paged_attention(
     float scale,
     int window, int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
     int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, int tiles_per_workgroup,
-    int merge_in_workgroup, int tile_halves, const float* sinks, hipStream_t stream) {
+    int merge_in_workgroup, int tile_halves, const float* sinks, float softcap, hipStream_t stream) {
     if (n_items <= 0 && n_tiles <= 0) return 0;
+    if (softcap < 0.f) return -1;
     // decode_fusion (see DecodeFusion::mode): the caller promises that every row of the step brings one token.
     DecodeFusion fusion = {q_weight, k_weight, cos_sin, norm_eps, decode_fusion};
     if (decode_fusion != 0 && decode_fusion != 1 && decode_fusion != 3) return -1;
@@ -1414,6 +1433,7 @@ LSA_EXPORT int lsa_paged_attention(
     Geometry g;
     g.n_q = n_q; g.n_kv = n_kv; g.group = n_q / n_kv; g.gheads = gheads; g.tokens_per_tile = tokens_per_tile;
     g.gtiles = gtiles; g.page_size = page_size; g.window = window; g.scale = scale; g.sinks = sinks;
+    g.cap = softcap; g.cap_inverse = softcap > 0.f ? 1.f / softcap : 0.f; g.scale_inverse = scale != 0.f ? 1.f / scale : 0.f;
     g.page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if (n_tiles > 0) {
 #if LSA_BF16

@@ -173,8 +173,15 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
 }
 
 // ------------------------------------------------------------------------------------------
-// SwiGLU: out[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g * sigmoid(g).
-template <typename T, int V>
+// Gated activation: out[t, i] = act(gu[t, i]) * gu[t, I + i]; act 0: silu(g) = g * sigmoid(g); act 1: the tanh form of
+// GELU, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
+template <int ACT>
+__device__ __forceinline__ float gate_activation(float g) {
+    if (ACT == 1) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.f + expf(-g));
+}
+
+template <typename T, int V, int ACT>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter) {
     const int t = blockIdx.y;
     const int i = (blockIdx.x * blockDim.x + threadIdx.x) * V;
@@ -187,12 +194,12 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             const float gv = (float)a.v[k];
-            r.v[k] = (T)(gv / (1.f + expf(-gv)) * (float)b.v[k]);
+            r.v[k] = (T)(gate_activation<ACT>(gv) * (float)b.v[k]);
         }
         store_vec16(o, r);
     } else {
         const float gv = (float)g[0];
-        o[0] = (T)(gv / (1.f + expf(-gv)) * (float)u[0]);
+        o[0] = (T)(gate_activation<ACT>(gv) * (float)u[0]);
     }
 }
 
@@ -233,16 +240,16 @@ static int launch_add_rmsnorm(void* resid, const void* delta, PartialSums partia
     LSA_LAUNCH_CHECK();
 }
 
-template <typename T>
+template <typename T, int ACT>
 static int launch_swiglu(const void* gate_up, void* out, int n_tokens, int inter, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (inter % Elem<T>::kVec == 0) {
         constexpr int V = Elem<T>::kVec;
         dim3 grid((inter / V + 255) / 256, n_tokens);
-        swiglu_kernel<T, V><<<grid, 256, 0, stream>>>((const T*)gate_up, (T*)out, inter);
+        swiglu_kernel<T, V, ACT><<<grid, 256, 0, stream>>>((const T*)gate_up, (T*)out, inter);
     } else {
         dim3 grid((inter + 255) / 256, n_tokens);
-        swiglu_kernel<T, 1><<<grid, 256, 0, stream>>>((const T*)gate_up, (T*)out, inter);
+        swiglu_kernel<T, 1, ACT><<<grid, 256, 0, stream>>>((const T*)gate_up, (T*)out, inter);
     }
     LSA_LAUNCH_CHECK();
 }
@@ -276,9 +283,12 @@ LSA_EXPORT int lsa_add_rmsnorm_partial_sums(int dtype, void* resid, const float*
     return dtype ? launch_add_rmsnorm<bf16_t>(resid, nullptr, partial, weight, eps, out, rows, n_out, width, stream)
                  : launch_add_rmsnorm<float>(resid, nullptr, partial, weight, eps, out, rows, n_out, width, stream);
 }
-LSA_EXPORT int lsa_swiglu(int dtype, const void* gate_up, void* out, int n_tokens, int inter, hipStream_t stream) {
-    return dtype ? launch_swiglu<bf16_t>(gate_up, out, n_tokens, inter, stream)
-                 : launch_swiglu<float>(gate_up, out, n_tokens, inter, stream);
+LSA_EXPORT int lsa_swiglu(int dtype, const void* gate_up, void* out, int n_tokens, int inter, int activation, hipStream_t stream) {
+    if (activation == 1)
+        return dtype ? launch_swiglu<bf16_t, 1>(gate_up, out, n_tokens, inter, stream) : launch_swiglu<float, 1>(gate_up, out, n_tokens, inter, stream);
+    if (activation != 0) return -1;
+    return dtype ? launch_swiglu<bf16_t, 0>(gate_up, out, n_tokens, inter, stream)
+                 : launch_swiglu<float, 0>(gate_up, out, n_tokens, inter, stream);
 }
 LSA_EXPORT int lsa_add_bias(int dtype, void* y, const float* bias, int n_tokens, int n, hipStream_t stream) {
     return dtype ? launch_add_bias<bf16_t>(y, bias, n_tokens, n, stream)

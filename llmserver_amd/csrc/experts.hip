@@ -9,6 +9,17 @@ using namespace lsa;
 
 constexpr float NEG_INF = -__builtin_huge_valf();
 
+// The experts' activation.  limit <= 0: silu(gate) * up.  limit > 0: the clamped form g * sigmoid(1.702 g) * (u + 1) with
+// g = min(gate, limit), u = clamp(up, -limit, limit).
+__device__ __forceinline__ float gated_activation(float g, float u, float limit) {
+    if (limit > 0.f) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+    }
+    return g / (1.f + expf(-g)) * u;
+}
+
 // Dot product of a weight row with a vector in LDS, a wavefront wide: 16-byte pieces where the length allows.
 template <typename T>
 __device__ inline float wave_dot(const T* __restrict__ w, const T* x_lds, int n, int lane) {
@@ -79,13 +90,50 @@ __global__ __launch_bounds__(256) void route_logits_kernel(const float* __restri
 // of experts lane, lane + 64, ... in LDS (its own entries only: nothing crosses lanes through LDS), and every lane ends
 // each round with the same (best, where).
 __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict__ all_logits, int experts, int top,
-                                                        int* __restrict__ chosen, float* __restrict__ weights, int n_tokens) {
+                                                        int* __restrict__ chosen, float* __restrict__ weights, int n_tokens,
+                                                        int sigmoid_scores, int groups, int keep) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = blockIdx.x * (blockDim.x >> 6) + wave;
     if (t >= n_tokens) return;
-    float* logits = lds + (size_t)wave * experts;
-    for (int e = lane; e < experts; e += 64) logits[e] = all_logits[(size_t)t * experts + e];
+    // (two arrays a wavefront: the values the choice is made among, and, for sigmoid scores, the scores themselves)
+    float* logits = lds + (size_t)wave * 2 * experts;
+    float* scores = logits + experts;
+    for (int e = lane; e < experts; e += 64) {
+        float v = all_logits[(size_t)t * experts + e];
+        if (sigmoid_scores) v = 1.f / (1.f + expf(-v));
+        logits[e] = v;
+        scores[e] = v;
+    }
+    if (sigmoid_scores && groups > 1) {
+        // A group's score is the sum of its two largest scores; the `keep` best groups stay (the first of equal ones),
+        // the experts of the others cannot be chosen.  Lane g (and g + 64, ...) scores group g; entries of other lanes
+        // are read here (a wavefront's LDS operations complete in the order they were issued).
+        __builtin_amdgcn_wave_barrier();
+        const int per = experts / groups;
+        {
+            const int base = 0, g = lane;             // (at most 64 groups: the host refuses more)
+            float mine = NEG_INF;
+            if (g < groups) {
+                float first = NEG_INF, second = NEG_INF;
+                for (int i = 0; i < per; ++i) {
+                    const float v = scores[g * per + i];
+                    if (v > first) { second = first; first = v; }
+                    else if (v > second) second = v;
+                }
+                mine = per > 1 ? first + second : first;
+            }
+            // rank of my group among all: groups with a larger score, or an equal one and a smaller index, come first
+            int before = 0;
+            for (int other = 0; other < min(64, groups - base); ++other) {
+                const float theirs = __shfl(mine, other, 64);
+                before += (theirs > mine || (theirs == mine && other < lane)) ? 1 : 0;
+            }
+            if (g < groups && before >= keep)
+                for (int i = 0; i < per; ++i) logits[g * per + i] = NEG_INF;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
     float largest = 0.f, total = 0.f;
     for (int k = 0; k < top; ++k) {
         float best = NEG_INF;
@@ -102,7 +150,7 @@ __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict_
         }
         if (where >= experts) where = k < experts ? k : 0;        // (only if every logit left is NaN or -inf)
         if (k == 0) largest = best;
-        const float weight = expf(best - largest);
+        const float weight = sigmoid_scores ? best : expf(best - largest);
         total += weight;
         if (lane == 0) {
             chosen[(size_t)t * top + k] = where;
@@ -110,7 +158,7 @@ __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict_
         }
         if ((where & 63) == lane) logits[where] = NEG_INF;
     }
-    if (lane == 0)
+    if (lane == 0 && !sigmoid_scores)
         for (int k = 0; k < top; ++k) weights[(size_t)t * top + k] /= total;         // (its own writes)
 }
 
@@ -118,7 +166,8 @@ __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict_
 template <typename T>
 __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ gate_up,
                                                               const int* __restrict__ chosen, T* __restrict__ hidden, int top,
-                                                              int inter, int width, int experts, int columns_per_block, bool in_lds) {
+                                                              int inter, int width, int experts, int columns_per_block, bool in_lds,
+                                                              float limit) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
     const int pair = blockIdx.x, t = pair / top;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
@@ -136,7 +185,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
     for (int f = f0 + wave; f < f1; f += waves) {
         float g, u;
         wave_dot2(base + (size_t)f * width, base + (size_t)(inter + f) * width, x_lds, width, lane, g, u);
-        if (lane == 0) hidden[(size_t)pair * inter + f] = (T)(g / (1.f + expf(-g)) * u);
+        if (lane == 0) hidden[(size_t)pair * inter + f] = (T)gated_activation(g, u, limit);
     }
 }
 
@@ -208,23 +257,28 @@ LSA_EXPORT int lsa_route_logits(const float* x, const float* router, float* logi
     LSA_LAUNCH_CHECK();
 }
 
-LSA_EXPORT int lsa_route_top(const float* logits, int experts, int top, int* chosen, float* weights, int n, hipStream_t stream) {
+// sigmoid_scores: the choice is made among sigmoid(logits), which are the weights as they are; groups > 1: only the
+// experts of the `keep` best of `groups` equal groups of neighbours can be chosen (at most 64 groups).
+LSA_EXPORT int lsa_route_top(const float* logits, int experts, int top, int* chosen, float* weights, int n, int sigmoid_scores,
+                             int groups, int keep, hipStream_t stream) {
     if (n <= 0) return 0;
-    if (top < 1 || top > experts || (size_t)experts * 16 > 60000) return -1;
-    route_top_kernel<<<(n + 3) / 4, 256, (size_t)experts * 4 * sizeof(float), stream>>>(logits, experts, top, chosen, weights, n);
+    if (top < 1 || top > experts || (size_t)experts * 32 > 60000) return -1;
+    if (groups > 1 && (!sigmoid_scores || groups > 64 || experts % groups || keep < 1 || keep > groups || top > keep * (experts / groups))) return -1;
+    route_top_kernel<<<(n + 3) / 4, 256, (size_t)experts * 8 * sizeof(float), stream>>>(logits, experts, top, chosen, weights, n,
+                                                                                       sigmoid_scores, groups, keep);
     LSA_LAUNCH_CHECK();
 }
 
 LSA_EXPORT int lsa_experts_gate_up(int code, const void* x, const void* gate_up, const int* chosen, void* hidden, int n, int top,
-                                   int inter, int width, int experts, hipStream_t stream) {
+                                   int inter, int width, int experts, float limit, hipStream_t stream) {
     if (n <= 0) return 0;
     size_t lds = (size_t)width * (code ? 2 : 4);
     const bool in_lds = lds <= 64000;
     if (!in_lds) lds = 0;
     const int columns = 16;
     dim3 grid(n * top, (inter + columns - 1) / columns);
-    if (code) experts_gate_up_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, chosen, (bf16_t*)hidden, top, inter, width, experts, columns, in_lds);
-    else experts_gate_up_kernel<float><<<grid, 256, lds, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)hidden, top, inter, width, experts, columns, in_lds);
+    if (code) experts_gate_up_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, chosen, (bf16_t*)hidden, top, inter, width, experts, columns, in_lds, limit);
+    else experts_gate_up_kernel<float><<<grid, 256, lds, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)hidden, top, inter, width, experts, columns, in_lds, limit);
     LSA_LAUNCH_CHECK();
 }
 
@@ -297,7 +351,7 @@ template <int BK, bool GATED, typename O, int NT>
 __global__ __launch_bounds__(256) void experts_tile_kernel(const bf16_t* __restrict__ a, int a_stride, int pair_div,
                                                            const bf16_t* __restrict__ b, long expert_stride, int b_rows, int b_up_offset,
                                                            const int* __restrict__ sorted, const int* __restrict__ tile_expert,
-                                                           O* __restrict__ out, int out_stride, int n_out, int k) {
+                                                           O* __restrict__ out, int out_stride, int n_out, int k, float limit) {
     constexpr int ROW = BK + 8;                                    // elements of a padded row in LDS
     __shared__ __align__(16) bf16_t a_lds[TILE_M * ROW];
     constexpr int BN = 32 * NT;                                    // rows of B a block takes
@@ -397,7 +451,7 @@ __global__ __launch_bounds__(256) void experts_tile_kernel(const bf16_t* __restr
                 for (int j = 0; j < NT / 2; ++j) {
                     const int f = n0 + wave_n * (BN / 4) + 16 * j + col;
                     const float g = acc[i][j][r], u = acc[i][j + NT / 2][r];
-                    if (f < n_out) o[f] = (O)(g / (1.f + expf(-g)) * u);
+                    if (f < n_out) o[f] = (O)gated_activation(g, u, limit);
                 }
             } else {
 #pragma unroll
@@ -426,7 +480,7 @@ LSA_EXPORT int lsa_experts_tile_rows() { return TILE_M; }
 // Scratch: sorted [max_tiles * 64] and tile_expert [max_tiles] ints, y [pairs, width] floats; max_tiles >= ceil(pairs / 64) + experts.
 LSA_EXPORT int lsa_experts_tiled(const void* x, const void* gate_up, const void* down, const int* chosen, const float* weights,
                                  void* hidden, float* y, float* out, int* sorted, int* tile_expert, int max_tiles, int n, int top,
-                                 int inter, int width, int experts, hipStream_t stream) {
+                                 int inter, int width, int experts, float limit, hipStream_t stream) {
     if (n <= 0) return 0;
     const int pairs = n * top;
     if (width % 32 || inter % 32 || max_tiles < (pairs + TILE_M - 1) / TILE_M + experts || (size_t)experts * 8 > 60000) return -1;
@@ -438,8 +492,8 @@ LSA_EXPORT int lsa_experts_tiled(const void* x, const void* gate_up, const void*
     const bool many = pairs >= 16 * experts;                    // pairs to an expert: wide tiles pay
 #define LSA_TILES(BK, NT) do { \
         dim3 grid1(max_tiles, (inter + 16 * NT - 1) / (16 * NT)), grid2(max_tiles, (width + 32 * NT - 1) / (32 * NT)); \
-        if (!second) experts_tile_kernel<BK, true, bf16_t, NT><<<grid1, 256, 0, stream>>>(xb, width, top, gu, (long)2 * inter * width, 2 * inter, inter, sorted, tile_expert, hb, inter, inter, width); \
-        else experts_tile_kernel<BK, false, float, NT><<<grid2, 256, 0, stream>>>(hb, inter, 1, dn, (long)width * inter, width, 0, sorted, tile_expert, y, width, width, inter); \
+        if (!second) experts_tile_kernel<BK, true, bf16_t, NT><<<grid1, 256, 0, stream>>>(xb, width, top, gu, (long)2 * inter * width, 2 * inter, inter, sorted, tile_expert, hb, inter, inter, width, limit); \
+        else experts_tile_kernel<BK, false, float, NT><<<grid2, 256, 0, stream>>>(hb, inter, 1, dn, (long)width * inter, width, 0, sorted, tile_expert, y, width, width, inter, 0.f); \
     } while (0)
     for (int pass = 0; pass < 2; ++pass) {
         const bool second = pass == 1;

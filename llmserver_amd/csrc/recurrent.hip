@@ -1,0 +1,258 @@
+// Kernels of the mixers that carry a state of fixed size from token to token: the mix of a token's row with the row
+// before it, the linear recurrence S_t = diag(d_t) S_(t-1) + k_t v_t^T with its read-out, and the per-head norm and gate
+// behind it.  Decays, their exponentials and logarithms, the state, the sums and the norm are float32; projections
+// arrive in the activations' type and are widened where they are read; a result for a 16-bit consumer is rounded once.
+#include "common.hpp"
+
+using namespace lsa;
+
+// out[m][t] = h[t] + (before[t] - h[t]) * mu[m], before[t] = the row of the token before t in its request: a row of this
+// step, the request's state for a row's first token, zeros at position 0.  One workgroup per token.  keep (only in
+// steps of one token per row, where a row's state is one workgroup's): the state becomes this token's row.
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_kernel(const T* __restrict__ h, const float* __restrict__ mu, int mixes,
+                                                          float* state, long state_stride, const int* __restrict__ slots,
+                                                          const int* __restrict__ token_row, const int* __restrict__ positions,
+                                                          const int* __restrict__ row_start, T* __restrict__ out, int n_tokens, int width,
+                                                          int keep) {
+    const int t = blockIdx.x;
+    const int row = token_row[t];
+    const bool first_of_sequence = positions[t] == 0, first_of_row = t == row_start[row];
+    float* mine = state + (size_t)slots[row] * state_stride;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const float own = (float)h[(size_t)t * width + c];
+        float before = 0.f;
+        if (!first_of_sequence) before = first_of_row ? mine[c] : (float)h[(size_t)(t - 1) * width + c];
+        const float difference = before - own;
+        for (int m = 0; m < mixes; ++m)
+            out[((size_t)m * n_tokens + t) * width + c] = (T)(own + difference * mu[(size_t)m * width + c]);
+        if (keep) mine[c] = own;
+    }
+}
+
+// state[slot] = the last row of every row of the step (rows without tokens keep theirs).
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_keep_kernel(const T* __restrict__ h, float* __restrict__ state, long state_stride,
+                                                               const int* __restrict__ slots, const int* __restrict__ row_start,
+                                                               const int* __restrict__ row_len, int width) {
+    const int row = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    const int count = row_len[row];
+    if (c >= width || count <= 0) return;
+    state[(size_t)slots[row] * state_stride + c] = (float)h[(size_t)(row_start[row] + count - 1) * width + c];
+}
+
+// The decay of a key channel from its 32-bit logit.  mode 0: sigmoid(z)^(1 / tau) = exp(log sigmoid(z) / tau);
+// mode 1: exp(-exp(z)).
+__device__ __forceinline__ float decay_of(float z, int mode, float inv_tau) {
+    if (mode == 0) {
+        const float log_sigmoid = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+        return expf(log_sigmoid * inv_tau);
+    }
+    return expf(-expf(z));
+}
+
+// grid (rows, heads, blocks of 64 value columns); a workgroup of NW wavefronts walks the row's tokens in order.
+// Lane = value column; wavefront w owns key channels [w * DK, (w + 1) * DK) and keeps its DK x 64 piece of the head's
+// state in registers, so the state is read once before the row's first token and written once after its last one.
+// The tokens go through LDS in chunks of CHUNK: queries (scaled), keys and decays of the head, widened and, for the
+// decays, exponentiated once per (token, channel) by whichever thread loads them; the chunk's values of this block of
+// columns; and, per wavefront, the partial read-outs of its channels, which are added up over the wavefronts when the
+// chunk is through.  A wavefront reads its channels of a token from LDS as broadcasts; nothing crosses lanes.
+//   BONUS false: S = d S + k v^T, then o = S^T q.      BONUS true: o = (S + (u k) v^T)^T q, then S = d S + k v^T.
+// Every sum is formed in the same order whatever the step's other rows and however the sequence was cut into steps:
+// the state after a token and the token's read-out are the same bits either way.
+constexpr int CHUNK = 16;
+
+template <typename T, int DK, bool BONUS>
+__global__ void linear_recurrence_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
+                                         const T* __restrict__ v, long v_stride, const float* __restrict__ decay,
+                                         const float* __restrict__ decay_bias, int mode, float inv_tau, const float* __restrict__ bonus,
+                                         float q_scale, float* state, long state_stride, const int* __restrict__ slots,
+                                         const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+                                         float* __restrict__ out, int heads, int dim, int value_dim) {
+    extern __shared__ __align__(16) float lds[];
+    const int row = blockIdx.x, head = blockIdx.y, column0 = blockIdx.z * 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int count = row_len[row];
+    if (count <= 0) return;                              // (the whole workgroup: nobody waits at a barrier below)
+    const int start = row_start[row], first_position = row_ctx[row] - count;
+    const int padded = waves * DK;                       // channels as the wavefronts share them; those behind dim are zeros
+    float* s_q = lds;                                    // [CHUNK][padded]
+    float* s_k = s_q + CHUNK * padded;
+    float* s_d = s_k + CHUNK * padded;
+    float* s_v = s_d + CHUNK * padded;                   // [CHUNK][64]
+    float* s_o = s_v + CHUNK * 64;                       // [waves][CHUNK][64]
+    const int column = column0 + lane;
+    const bool column_ok = column < value_dim;
+    const int channel0 = wave * DK;
+    float* mine = state + (size_t)slots[row] * state_stride + ((size_t)head * dim + channel0) * value_dim + column;
+    float S[DK], u[DK];
+#pragma unroll
+    for (int i = 0; i < DK; ++i) {
+        const bool ok = column_ok && channel0 + i < dim;
+        S[i] = (ok && first_position > 0) ? mine[(size_t)i * value_dim] : 0.f;
+        u[i] = (BONUS && channel0 + i < dim) ? bonus[(size_t)head * dim + channel0 + i] : 0.f;
+    }
+    const size_t key_column = (size_t)head * dim;
+    for (int t0 = 0; t0 < count; t0 += CHUNK) {
+        const int n = min(CHUNK, count - t0);
+        __syncthreads();                                 // the chunk before has been read out of LDS
+        for (int i = threadIdx.x; i < n * padded; i += blockDim.x) {
+            const int t = i / padded, c = i - t * padded;
+            const size_t token = (size_t)(start + t0 + t);
+            float qv = 0.f, kv = 0.f, dv = 1.f;
+            if (c < dim) {
+                qv = (float)q[token * q_stride + key_column + c] * q_scale;
+                kv = (float)k[token * k_stride + key_column + c];
+                const float z = decay[token * (size_t)heads * dim + key_column + c] + (decay_bias ? decay_bias[key_column + c] : 0.f);
+                dv = decay_of(z, mode, inv_tau);
+            }
+            s_q[i] = qv;
+            s_k[i] = kv;
+            s_d[i] = dv;
+        }
+        for (int i = threadIdx.x; i < n * 64; i += blockDim.x) {
+            const int t = i >> 6, c = column0 + (i & 63);
+            s_v[i] = c < value_dim ? (float)v[(size_t)(start + t0 + t) * v_stride + (size_t)head * value_dim + c] : 0.f;
+        }
+        __syncthreads();
+        for (int t = 0; t < n; ++t) {
+            const float value = s_v[t * 64 + lane];
+            const float* tq = s_q + t * padded + channel0;
+            const float* tk = s_k + t * padded + channel0;
+            const float* td = s_d + t * padded + channel0;
+            float o = 0.f;
+#pragma unroll
+            for (int i = 0; i < DK; ++i) {
+                const float kv = tk[i] * value;
+                if (BONUS) {
+                    o = __builtin_fmaf(__builtin_fmaf(u[i], kv, S[i]), tq[i], o);
+                    S[i] = __builtin_fmaf(td[i], S[i], kv);
+                } else {
+                    S[i] = __builtin_fmaf(td[i], S[i], kv);
+                    o = __builtin_fmaf(S[i], tq[i], o);
+                }
+            }
+            s_o[(wave * CHUNK + t) * 64 + lane] = o;
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < n * 64; i += blockDim.x) {
+            const int t = i >> 6, c = i & 63;
+            if (column0 + c >= value_dim) continue;
+            float total = 0.f;
+            for (int w = 0; w < waves; ++w) total += s_o[(w * CHUNK + t) * 64 + c];
+            out[(size_t)(start + t0 + t) * heads * value_dim + (size_t)head * value_dim + column0 + c] = total;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DK; ++i)
+        if (column_ok && channel0 + i < dim) mine[(size_t)i * value_dim] = S[i];
+}
+
+// grid (tokens, heads), one wavefront: out = x / rms(x) * w * silu(gate) over a head's value_dim numbers; x float32,
+// w = weight[head * weight_stride + j] (weight_stride 0: one weight shared by the heads), gate and out of type T.
+template <typename T>
+__global__ __launch_bounds__(64) void heads_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ weight, int weight_stride,
+                                                             float eps, const T* __restrict__ gate, long gate_stride, T* __restrict__ out,
+                                                             int heads, int value_dim) {
+    const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const float* row = x + ((size_t)t * heads + head) * value_dim;
+    float sq = 0.f;
+    for (int j = lane; j < value_dim; j += 64) sq += row[j] * row[j];
+    const float inv = rsqrtf(wave_sum(sq) / (float)value_dim + eps);
+    const T* g = gate + (size_t)t * gate_stride + (size_t)head * value_dim;
+    const float* w = weight + (size_t)head * weight_stride;
+    T* o = out + ((size_t)t * heads + head) * value_dim;
+    for (int j = lane; j < value_dim; j += 64) {
+        const float gv = (float)g[j];
+        o[j] = (T)(row[j] * inv * w[j] * (gv / (1.f + expf(-gv))));
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tanh_kernel(T* __restrict__ x, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = (T)tanhf((float)x[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void scaled_sum_kernel(const T* __restrict__ x, float a, const T* __restrict__ y, float b,
+                                                         T* __restrict__ out, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (T)(a * (float)x[i] + b * (float)y[i]);
+}
+
+LSA_EXPORT int lsa_token_shift(int code, const void* h, const float* mu, int mixes, float* state, long state_stride, const int* slots,
+                               const int* token_row, const int* positions, const int* row_start, void* out, int n_tokens, int width,
+                               int keep, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (mixes < 1 || state == nullptr || slots == nullptr) return -1;
+#define LSA_LAUNCH(T) token_shift_kernel<T><<<n_tokens, 256, 0, stream>>>((const T*)h, mu, mixes, state, state_stride, slots, token_row, positions, \
+        row_start, (T*)out, n_tokens, width, keep)
+    if (code) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
+#undef LSA_LAUNCH
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_token_shift_keep(int code, const void* h, float* state, long state_stride, const int* slots, const int* row_start,
+                                    const int* row_len, int rows, int width, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    dim3 grid(rows, (width + 255) / 256);
+    if (code) token_shift_keep_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, state, state_stride, slots, row_start, row_len, width);
+    else token_shift_keep_kernel<float><<<grid, 256, 0, stream>>>((const float*)h, state, state_stride, slots, row_start, row_len, width);
+    LSA_LAUNCH_CHECK();
+}
+
+// Key channels a wavefront takes: 8 for heads of up to 64 channels, 16 up to 256, 32 up to 512 (at most 16 wavefronts).
+LSA_EXPORT int lsa_linear_recurrence_most_dim() { return 512; }
+
+LSA_EXPORT int lsa_linear_recurrence(int code, const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                                     const float* decay, const float* decay_bias, int mode, float tau, const float* bonus, float q_scale,
+                                     float* state, long state_stride, const int* slots, const int* row_start, const int* row_len,
+                                     const int* row_ctx, float* out, int rows, int heads, int dim, int value_dim, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dim < 1 || dim > 512 || value_dim < 1 || heads < 1 || (mode != 0 && mode != 1) || !(tau > 0.f) || state == nullptr) return -1;
+    const int dk = dim <= 64 ? 8 : dim <= 256 ? 16 : 32;
+    const int waves = (dim + dk - 1) / dk;
+    const size_t lds = sizeof(float) * ((size_t)3 * CHUNK * waves * dk + (size_t)CHUNK * 64 + (size_t)waves * CHUNK * 64);
+    dim3 grid(rows, heads, (value_dim + 63) / 64);
+#define LSA_LAUNCH(T, DK, B) do { \
+        if (lds > 48 * 1024) \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_recurrence_kernel<T, DK, B>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+        linear_recurrence_kernel<T, DK, B><<<grid, waves * 64, lds, stream>>>((const T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, \
+            decay, decay_bias, mode, 1.f / tau, bonus, q_scale, state, state_stride, slots, row_start, row_len, row_ctx, out, heads, dim, value_dim); \
+    } while (0)
+#define LSA_BY_DK(T, B) do { if (dk == 8) LSA_LAUNCH(T, 8, B); else if (dk == 16) LSA_LAUNCH(T, 16, B); else LSA_LAUNCH(T, 32, B); } while (0)
+    if (code) { if (bonus) LSA_BY_DK(bf16_t, true); else LSA_BY_DK(bf16_t, false); }
+    else { if (bonus) LSA_BY_DK(float, true); else LSA_BY_DK(float, false); }
+#undef LSA_BY_DK
+#undef LSA_LAUNCH
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_heads_norm_gate(int code, const float* x, const float* weight, int weight_per_channel, float eps, const void* gate,
+                                   long gate_stride, void* out, int n_tokens, int heads, int value_dim, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    dim3 grid(n_tokens, heads);
+    const int weight_stride = weight_per_channel ? value_dim : 0;
+    if (code) heads_norm_gate_kernel<bf16_t><<<grid, 64, 0, stream>>>(x, weight, weight_stride, eps, (const bf16_t*)gate, gate_stride, (bf16_t*)out, heads, value_dim);
+    else heads_norm_gate_kernel<float><<<grid, 64, 0, stream>>>(x, weight, weight_stride, eps, (const float*)gate, gate_stride, (float*)out, heads, value_dim);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_tanh(int code, void* x, long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    const int blocks = (int)((n + 255) / 256);
+    if (code) tanh_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, n);
+    else tanh_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, n);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_scaled_sum(int code, const void* x, float a, const void* y, float b, void* out, long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    const int blocks = (int)((n + 255) / 256);
+    if (code) scaled_sum_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)x, a, (const bf16_t*)y, b, (bf16_t*)out, n);
+    else scaled_sum_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, a, (const float*)y, b, (float*)out, n);
+    LSA_LAUNCH_CHECK();
+}

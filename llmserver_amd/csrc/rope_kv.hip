@@ -267,3 +267,71 @@ LSA_EXPORT int lsa_qk_norm_rope_kv_write(int dtype, void* qkv, void* keys, void*
                  : launch<float>(qkv, keys, values, table, table_stride, token_row, positions, q_weight, k_weight, eps,
                                  cos_sin, page_size, n_q, n_kv, d, write_cache, n_tokens, stream);
 }
+
+// ------------------------------------------------------------------------------------------
+// The general way of preparing queries, keys and values: heads of any size, values of another size than the keys,
+// a rotation of neighbouring pairs (2i, 2i + 1) on the first 2 * pairs dimensions of a head, rows filled up with zeros
+// to the head size D of the pages and the attention kernels.  grid (tokens, n_q + n_kv), one wavefront per (token,
+// head): a query head writes its row of out_q, a key/value head its key row and its value row (transposed) into the
+// token's place in the pages.  qkv row: n_q x dim queries, n_kv x dim keys, n_kv x value_dim values.
+template <typename T>
+__global__ __launch_bounds__(64) void qkv_prepare_kernel(const T* __restrict__ qkv, long stride, T* __restrict__ keys, T* __restrict__ values,
+                                                         const int* __restrict__ table, int table_stride, const int* __restrict__ token_row,
+                                                         const int* __restrict__ positions, const float* __restrict__ q_weight,
+                                                         const float* __restrict__ k_weight, float eps, const float* __restrict__ cos_sin,
+                                                         int pairs, int page_size, int n_q, int n_kv, int dim, int value_dim, int D,
+                                                         T* __restrict__ out_q, int write_cache) {
+    const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const bool is_query = head < n_q;
+    if (!is_query && !write_cache) return;
+    const T* src = qkv + (size_t)t * stride + (size_t)head * dim;             // (keys follow the queries, head by head)
+    const float* weight = is_query ? q_weight : k_weight;
+    float inv = 1.f;
+    if (weight) {
+        float sq = 0.f;
+        for (int e = lane; e < dim; e += 64) {
+            const float v = (float)src[e];
+            sq += v * v;
+        }
+        inv = rsqrtf(wave_sum(sq) / (float)dim + eps);
+    }
+    const float* cs = cos_sin ? cos_sin + (size_t)t * 2 * pairs : nullptr;
+    auto prepared = [&](int e) -> float {
+        if (e >= dim) return 0.f;
+        auto normed = [&](int i) { return weight ? (float)src[i] * inv * weight[i] : (float)src[i]; };
+        const int pair = e >> 1;
+        if (!cs || pair >= pairs) return normed(e);
+        const float u = normed(2 * pair), w = normed(2 * pair + 1), c = cs[pair], s = cs[pairs + pair];
+        return (e & 1) ? w * c + u * s : u * c - w * s;
+    };
+    if (is_query) {
+        T* o = out_q + ((size_t)t * n_q + head) * D;
+        for (int e = lane; e < D; e += 64) o[e] = (T)prepared(e);
+        return;
+    }
+    const int kv = head - n_q;
+    const int position = positions[t];
+    const int page = table[(size_t)token_row[t] * table_stride + position / page_size], slot = position % page_size;
+    if (page < 0) return;
+    T* key = keys + (((size_t)page * n_kv + kv) * page_size + slot) * D;
+    T* value = values + ((size_t)page * n_kv + kv) * D * page_size + slot;
+    const T* v = qkv + (size_t)t * stride + (size_t)(n_q + n_kv) * dim + (size_t)kv * value_dim;
+    for (int e = lane; e < D; e += 64) {
+        key[e] = (T)prepared(e);
+        value[(size_t)e * page_size] = e < value_dim ? v[e] : (T)0.f;
+    }
+}
+
+LSA_EXPORT int lsa_qkv_prepare(int dtype, const void* qkv, long stride, void* keys, void* values, const int* table, int table_stride,
+                               const int* token_row, const int* positions, const float* q_weight, const float* k_weight, float eps,
+                               const float* cos_sin, int pairs, int page_size, int n_q, int n_kv, int dim, int value_dim, int D,
+                               void* out_q, int write_cache, int n_tokens, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (dim > D || value_dim > D || 2 * pairs > dim || page_size <= 0 || (q_weight == nullptr) != (k_weight == nullptr)) return -1;
+    dim3 grid(n_tokens, n_q + n_kv);
+#define LSA_LAUNCH(T) qkv_prepare_kernel<T><<<grid, 64, 0, stream>>>((const T*)qkv, stride, (T*)keys, (T*)values, table, table_stride, token_row, \
+        positions, q_weight, k_weight, eps, cos_sin, pairs, page_size, n_q, n_kv, dim, value_dim, D, (T*)out_q, write_cache)
+    if (dtype) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
+#undef LSA_LAUNCH
+    LSA_LAUNCH_CHECK();
+}

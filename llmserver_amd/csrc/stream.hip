@@ -180,6 +180,116 @@ __global__ __launch_bounds__(256) void scaled_norm_add_kernel(const float* __res
     }
 }
 
+// out[t] = table[ids[t]] widened to float32 (an id outside the table gives a zero row).
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_wide_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                                             float* __restrict__ out, int width, int vocab) {
+    const int id = ids[blockIdx.x];
+    const bool ok = id >= 0 && id < vocab;
+    const T* row = table + (size_t)(ok ? id : 0) * width;
+    float* o = out + (size_t)blockIdx.x * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = ok ? (float)row[i] : 0.f;
+}
+
+// s = x + u * rsqrt(mean(u^2) + eps) * weight with u = y, or a * y + b * y2 where y2 is given; out = s; and where
+// next_weight is given, normed = s * rsqrt(mean(s^2) + next_eps) * next_weight: the norm behind a sublayer, the sum with
+// the stream and the norm in front of the next sublayer in one pass (the row stays in registers between the two sums
+// of squares; rows wider than 256 * V * CACHE elements are read again).
+template <typename Y, typename R, int V>
+__global__ __launch_bounds__(256) void norm_add_norm_kernel(const float* __restrict__ x, const Y* __restrict__ y, const Y* __restrict__ y2,
+                                                            float a, float b, const float* __restrict__ weight, float eps,
+                                                            float* __restrict__ out, const float* __restrict__ next_weight, float next_eps,
+                                                            R* __restrict__ normed, int width) {
+    constexpr int CACHE = 4;
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * width;
+    const int stride = blockDim.x * V;
+    auto update = [&](int i, float (&u)[V]) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) u[v] = y2 ? a * (float)y[base + i + v] + b * (float)y2[base + i + v] : (float)y[base + i + v];
+    };
+    float kept[CACHE][V];
+    float sq = 0.f;
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = threadIdx.x * V + k * stride;
+        if (i < width) {
+            update(i, kept[k]);
+#pragma unroll
+            for (int v = 0; v < V; ++v) sq += kept[k][v] * kept[k][v];
+        }
+    }
+    for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
+        float u[V];
+        update(i, u);
+#pragma unroll
+        for (int v = 0; v < V; ++v) sq += u[v] * u[v];
+    }
+    const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
+    float sq2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = threadIdx.x * V + k * stride;
+        if (i < width) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const float s = x[base + i + v] + kept[k][v] * inv * weight[i + v];
+                kept[k][v] = s;
+                out[base + i + v] = s;
+                sq2 += s * s;
+            }
+        }
+    }
+    for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
+        float u[V];
+        update(i, u);
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            const float s = x[base + i + v] + u[v] * inv * weight[i + v];
+            out[base + i + v] = s;
+            sq2 += s * s;
+        }
+    }
+    if (!next_weight) return;
+    const float inv2 = rsqrtf(block_sum(sq2, scratch) / (float)width + next_eps);
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = threadIdx.x * V + k * stride;
+        if (i < width) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) normed[base + i + v] = (R)(kept[k][v] * inv2 * next_weight[i + v]);
+        }
+    }
+    for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride)         // (its own writes of a moment ago)
+#pragma unroll
+        for (int v = 0; v < V; ++v) normed[base + i + v] = (R)(out[base + i + v] * inv2 * next_weight[i + v]);
+}
+
+LSA_EXPORT int lsa_embedding_wide(int table_code, const void* table, const int* ids, float* out, int n, int width, int vocab,
+                                  hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (table_code) embedding_wide_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)table, ids, out, width, vocab);
+    else embedding_wide_kernel<float><<<n, 256, 0, stream>>>((const float*)table, ids, out, width, vocab);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_norm_add_norm(const float* x, const void* y, const void* y2, int y_code, float a, float b, const float* weight, float eps,
+                                 float* out, const float* next_weight, float next_eps, void* normed, int normed_code, int n, int width,
+                                 hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (next_weight != nullptr && normed == nullptr) return -1;
+#define LSA_LAUNCH_V(Y, R, V) norm_add_norm_kernel<Y, R, V><<<n, 256, 0, stream>>>(x, (const Y*)y, (const Y*)y2, a, b, weight, eps, out, next_weight, \
+                                                                                next_eps, (R*)normed, width)
+#define LSA_LAUNCH(Y, R) do { if (width % 4 == 0) LSA_LAUNCH_V(Y, R, 4); else LSA_LAUNCH_V(Y, R, 1); } while (0)
+    if (y_code && normed_code) LSA_LAUNCH(bf16_t, bf16_t);
+    else if (y_code) LSA_LAUNCH(bf16_t, float);
+    else if (normed_code) LSA_LAUNCH(float, bf16_t);
+    else LSA_LAUNCH(float, float);
+#undef LSA_LAUNCH
+#undef LSA_LAUNCH_V
+    LSA_LAUNCH_CHECK();
+}
+
 LSA_EXPORT int lsa_embedding_norm(int table_code, const void* table, const int* ids, const float* weight, float eps, float* out,
                                   int n, int width, int vocab, hipStream_t stream) {
     if (n <= 0) return 0;

@@ -26,9 +26,9 @@ FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HEAD_DIMS = tuple(range(16, 257, 16))
 BASE_MODULES = ("elementwise", "rope_kv", "sampling", "gemm")
-# Libraries that only some models call (a 32-bit residual stream, attention over a latent, routed experts): loaded, and
-# compiled if need be, when the first such call is made.
-PART_MODULES = ("stream", "latent", "experts")
+# Libraries that only some models call (a 32-bit residual stream, attention over a latent, routed experts, mixers with a
+# recurrent state): loaded, and compiled if need be, when the first such call is made.
+PART_MODULES = ("stream", "latent", "experts", "recurrent")
 
 
 class KernelBuildError(RuntimeError):

@@ -12,7 +12,7 @@ _SIGNATURES = {
     "lsa_embedding": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_add_rmsnorm": [c_int, _P, _P, _P, c_float, _P, _P, c_int, c_int, _P],
     "lsa_add_rmsnorm_partial_sums": [c_int, _P, _P, c_int, c_long, _P, c_float, _P, _P, c_int, c_int, _P],
-    "lsa_swiglu": [c_int, _P, _P, c_int, c_int, _P],
+    "lsa_swiglu": [c_int, _P, _P, c_int, c_int, c_int, _P],
     "lsa_add_bias": [c_int, _P, _P, c_int, c_int, _P],
     "lsa_plain_read": [_P, _P, c_long, c_int, c_int, _P],
     "lsa_qk_norm_rope_kv_write": [c_int, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int,
@@ -24,7 +24,19 @@ _SIGNATURES = {
     "lsa_sample_static_max_rows": [],
     "lsa_sample_static_error": [c_int],
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, _P, c_int,
-                            c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P, _P],
+                            c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P, c_float, _P],
+    "lsa_embedding_wide": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_norm_add_norm": [_P, _P, _P, c_int, c_float, c_float, _P, c_float, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
+    "lsa_qkv_prepare": [c_int, _P, c_long, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                        _P, c_int, c_int, _P],
+    "lsa_token_shift": [c_int, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_token_shift_keep": [c_int, _P, _P, c_long, _P, _P, _P, c_int, c_int, _P],
+    "lsa_linear_recurrence_most_dim": [],
+    "lsa_linear_recurrence": [c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, c_float, _P, c_float, _P, c_long, _P, _P, _P, _P, _P,
+                              c_int, c_int, c_int, c_int, _P],
+    "lsa_heads_norm_gate": [c_int, _P, _P, c_int, c_float, _P, c_long, _P, c_int, c_int, c_int, _P],
+    "lsa_tanh": [c_int, _P, c_long, _P],
+    "lsa_scaled_sum": [c_int, _P, c_float, _P, c_float, _P, c_long, _P],
     "lsa_embedding_norm": [c_int, _P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_norm_rows": [_P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_short_conv": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
@@ -34,10 +46,10 @@ _SIGNATURES = {
                            c_int, c_int, c_int, c_int, _P],
     "lsa_gate_heads": [c_int, _P, _P, _P, c_int, c_int, _P, c_long, c_int, _P, c_int, c_int, c_int, _P],
     "lsa_route_logits": [_P, _P, _P, c_int, c_int, c_int, _P],
-    "lsa_route_top": [_P, c_int, c_int, _P, _P, c_int, _P],
-    "lsa_experts_gate_up": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    "lsa_route_top": [_P, c_int, c_int, _P, _P, c_int, c_int, c_int, c_int, _P],
+    "lsa_experts_gate_up": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P],
     "lsa_experts_tile_rows": [],
-    "lsa_experts_tiled": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+    "lsa_experts_tiled": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
     "lsa_experts_down": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_attention_workgroup_tiles": [],
     "lsa_attention_tile_page_multiple": [],

@@ -513,7 +513,8 @@ class HipOps(KernelNamespace):
                   "gemm_skinny_stream")
         return stream, weighted, square_sums
 
-    ACTIVATIONS = ("silu",)       # what the activation kernel and the gated products' epilogues compute
+    ACTIVATIONS = ("silu", "gelu_tanh")       # what the activation kernel computes (its codes are the places in this list)
+    FUSED_ACTIVATIONS = ("silu",)             # ... and what the gated products' epilogues compute
 
     def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None, activation="silu"):
         """``silu(x @ gate^T) * (x @ up^T)`` with ``gate_up_weight [2I, K]`` in one launch for few rows (the
@@ -522,7 +523,7 @@ class HipOps(KernelNamespace):
         ``row_scale`` as in :meth:`linear_few_rows`."""
         rows, width = x.shape
         inter = gate_up_weight.shape[0] // 2
-        if activation not in self.ACTIVATIONS:
+        if activation not in self.FUSED_ACTIVATIONS:
             return None
         if rows > self.skinny_rows:
             return self._linear_gated_beyond_few_rows(x, gate_up_weight) if row_scale is None and pairs_per_workgroup == 0 else None
@@ -597,7 +598,8 @@ class HipOps(KernelNamespace):
         n, inter = out.shape
         _check(gate_up, "gate_up", out.dtype, (n, 2 * inter))
         _check(out, "out")
-        _launched(self._elementwise.lsa_swiglu(_code(out), _ptr(gate_up), _ptr(out), n, inter, _stream()), "swiglu")
+        _launched(self._elementwise.lsa_swiglu(_code(out), _ptr(gate_up), _ptr(out), n, inter, self.ACTIVATIONS.index(activation), _stream()),
+                  "swiglu")
 
     def add_bias_(self, y, bias):
         n, width = y.shape
@@ -681,7 +683,7 @@ class HipOps(KernelNamespace):
         return dtype == torch.bfloat16 and head_dim % 64 == 0
 
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None, sinks=None, softcap=None):
         """Attention of the step's tokens over their requests' pages.
 
         ``qkv [T, (n_q + 2 n_kv) * d]`` holds the normalised, rotated queries in its first
@@ -693,7 +695,8 @@ class HipOps(KernelNamespace):
         ``write_cache``) takes the new key and value from ``qkv`` and puts them into the pages.
 
         Without ``decode_fusion``, ``qkv`` may hold the queries alone (``[T, n_q * d]``).  ``sinks [n_q]`` float32: one
-        more term ``exp(sinks[head])`` in the denominator of every softmax of that head (no key, no value).
+        more term ``exp(sinks[head])`` in the denominator of every softmax of that head (no key, no value).  ``softcap``: scaled
+        scores become ``softcap * tanh(score / softcap)`` before the mask.
         """
         n = qkv.shape[0]
         if decode_fusion is None and qkv.shape[1] == n_q * head_dim:
@@ -770,7 +773,7 @@ class HipOps(KernelNamespace):
             n_merges, n_slots, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), _ptr(tile_slots), n_tiles, float(scale), int(window) if window else 0,
             page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, fusion_mode, _ptr(q_weight), _ptr(k_weight), float(norm_eps),
             _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), merge_in_workgroup, int(plan.get("tile_halves", 1)), _ptr(sinks),
-            _stream()), "paged_attention")
+            float(softcap) if softcap else 0.0, _stream()), "paged_attention")
 
     # -- a residual stream in float32, attention over a latent, routed experts ---------------------------
     # (libraries of their own, loaded at the first call: models that have none of these parts never build them)
@@ -790,6 +793,34 @@ class HipOps(KernelNamespace):
             raise ValueError(f"embedding: table width {table.shape[1]} != out width {width}")
         _launched(self._part_library("stream").lsa_embedding_norm(_code(table), _ptr(table), _ptr(token_ids), _ptr(weight), float(eps),
                                                                   _ptr(out), n, width, table.shape[0], _stream()), "embedding_norm")
+
+    def embedding_wide(self, table, token_ids, out):
+        n, width = out.shape
+        _check(table, "table")
+        _check(token_ids, "token_ids", torch.int32, (n,))
+        _check(out, "out", torch.float32)
+        if table.shape[1] != width:
+            raise ValueError(f"embedding: table width {table.shape[1]} != out width {width}")
+        _launched(self._part_library("stream").lsa_embedding_wide(_code(table), _ptr(table), _ptr(token_ids), _ptr(out), n, width,
+                                                                  table.shape[0], _stream()), "embedding_wide")
+
+    def norm_add_norm(self, x, y, weight, eps, out, next_weight=None, next_eps=0.0, normed=None, y2=None, scales=None):
+        n, width = x.shape
+        _check(x, "x", torch.float32)
+        _check(y, "y", None, (n, width))
+        _check(weight, "weight", torch.float32, (width,))
+        _check(out, "out", torch.float32, (n, width))
+        a = b = 1.0
+        if y2 is not None:
+            _check(y2, "y2", y.dtype, (n, width))
+            a, b = (float(scale) for scale in scales)
+        if next_weight is not None:
+            _check(next_weight, "next_weight", torch.float32, (width,))
+            _check(normed, "normed", None, (n, width))
+        _launched(self._part_library("stream").lsa_norm_add_norm(
+            _ptr(x), _ptr(y), _ptr(y2), _code(y), a, b, _ptr(weight), float(eps), _ptr(out), _ptr(next_weight), float(next_eps),
+            _ptr(normed) if next_weight is not None else None, _code(normed) if next_weight is not None else 0, n, width, _stream()),
+            "norm_add_norm")
 
     def norm_rows(self, x, rows, weight, eps, out):
         n_out, width = out.shape
@@ -915,8 +946,8 @@ class HipOps(KernelNamespace):
         _launched(self._part_library("latent").lsa_gate_heads(_code(out), _ptr(y), _ptr(mixed), _ptr(up_values), rank, row_width, _ptr(proj),
                                                               proj.shape[1], int(gate_column), _ptr(out), heads, v, n, _stream()), "gate_heads")
 
-    def route_experts(self, x, router, top, chosen, weights):
-        """The logits are a float32 product of the library (no reduced-precision mode), the choice and the softmax a kernel."""
+    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None):
+        """The logits are a float32 product of the library (no reduced-precision mode), the choice and the weights a kernel."""
         n, width = x.shape
         experts = router.shape[0]
         _check(x, "x")
@@ -932,10 +963,24 @@ class HipOps(KernelNamespace):
                       "route_logits")
         else:
             logits = torch.mm(wide, router.t())
-        _launched(self._part_library("experts").lsa_route_top(_ptr(logits), experts, top, _ptr(chosen), _ptr(weights), n, _stream()),
-                  "route_top")
+        if scoring not in ("softmax", "sigmoid") or (groups is not None and scoring != "sigmoid"):
+            raise ValueError(f"the router kernel scores by softmax or sigmoid (groups with sigmoid only), asked for {scoring!r}, groups {groups}")
+        count, keep = groups if groups is not None else (1, 1)
+        if count > 64 or experts % count or not 1 <= keep <= count or top > keep * (experts // count):
+            raise ValueError(f"the router kernel takes up to 64 equal groups: {experts} experts in {count} groups, {keep} kept, {top} chosen")
+        _launched(self._part_library("experts").lsa_route_top(_ptr(logits), experts, top, _ptr(chosen), _ptr(weights), n,
+                                                              1 if scoring == "sigmoid" else 0, int(count), int(keep), _stream()), "route_top")
 
-    def experts_gate_up(self, x, gate_up, chosen, hidden):
+    @staticmethod
+    def _expert_limit(activation, limit) -> float:
+        """What the experts' kernels take for the activation: 0 for silu(gate) * up, the limit of the clamped form."""
+        if activation == "silu":
+            return 0.0
+        if activation != "clamped" or not limit > 0.0:
+            raise ValueError(f"the experts' kernels compute silu, or the clamped form with a positive limit; asked for {activation!r}, {limit}")
+        return float(limit)
+
+    def experts_gate_up(self, x, gate_up, chosen, hidden, activation="silu", limit=0.0):
         n, width = x.shape
         experts, top, inter = gate_up.shape[0], chosen.shape[1], hidden.shape[1]
         _check(x, "x")
@@ -943,7 +988,8 @@ class HipOps(KernelNamespace):
         _check(chosen, "chosen", torch.int32, (n, top))
         _check(hidden, "hidden", x.dtype, (n * top, inter))
         _launched(self._part_library("experts").lsa_experts_gate_up(_code(x), _ptr(x), _ptr(gate_up), _ptr(chosen), _ptr(hidden), n, top,
-                                                                    inter, width, experts, _stream()), "experts_gate_up")
+                                                                    inter, width, experts, self._expert_limit(activation, limit), _stream()),
+                  "experts_gate_up")
 
     def experts_down(self, hidden, down, chosen, weights, out):
         n, width = out.shape
@@ -956,7 +1002,7 @@ class HipOps(KernelNamespace):
         _launched(self._part_library("experts").lsa_experts_down(_code(hidden), _ptr(hidden), _ptr(down), _ptr(chosen), _ptr(weights),
                                                                  _ptr(out), n, top, inter, width, experts, _stream()), "experts_down")
 
-    def experts_sorted(self, x, gate_up, down, chosen, weights, out) -> bool:
+    def experts_sorted(self, x, gate_up, down, chosen, weights, out, activation="silu", limit=0.0) -> bool:
         """Offered in bfloat16 for widths and expert sizes in steps of 32, and taken where the step has more (token,
         expert) pairs than there are experts: below that every pair streaming its own expert reads no more."""
         n, width = x.shape
@@ -977,8 +1023,128 @@ class HipOps(KernelNamespace):
         scratch = torch.empty((max_tiles * (tile + 1),), device=x.device, dtype=torch.int32)
         _launched(lib.lsa_experts_tiled(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(hidden), _ptr(y), _ptr(out),
                                         _ptr(scratch), scratch[max_tiles * tile:].data_ptr(), max_tiles, n, top, inter, width, experts,
-                                        _stream()), "experts_tiled")
+                                        self._expert_limit(activation, limit), _stream()), "experts_tiled")
         return True
+
+    # -- general preparation of queries, keys and values; mixers with a recurrent state -----------------------------
+    def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True):
+        n = qkv.shape[0]
+        _check(qkv, "qkv", None, (n, (n_q + n_kv) * dim + n_kv * value_dim))
+        pages, row = keys.shape[0], keys.shape[-1]
+        _check(keys, "keys", qkv.dtype, (pages, n_kv, page_size, row))
+        _check(values, "values", qkv.dtype, (pages, n_kv, row, page_size))
+        if dim > row or value_dim > row:
+            raise ValueError(f"heads of {dim} / {value_dim} do not fit the pages' rows of {row}")
+        _check(table, "table", torch.int32)
+        _check(token_row, "token_row", torch.int32, (n,))
+        _check(positions, "positions", torch.int32, (n,))
+        _check(out_q, "out_q", qkv.dtype, (n, n_q * row))
+        if (q_weight is None) != (k_weight is None):
+            raise ValueError("q and k norm weights must come together")
+        for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+            if w is not None:
+                _check(w, name, torch.float32, (dim,))
+        pairs = 0
+        if cos_sin is not None:
+            pairs = cos_sin.shape[1] // 2
+            _check(cos_sin, "cos_sin", torch.float32, (n, 2 * pairs))
+            if 2 * pairs > dim:
+                raise ValueError(f"{2 * pairs} dimensions turn, a head has {dim}")
+        _launched(self._rope_kv.lsa_qkv_prepare(
+            _code(qkv), _ptr(qkv), qkv.shape[1], _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions),
+            _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), pairs, page_size, n_q, n_kv, dim, value_dim, row, _ptr(out_q),
+            1 if write_cache else 0, n, _stream()), "qkv_prepare")
+
+    @staticmethod
+    def _state_rows(state, offset, needed, name):
+        """(pointer to column ``offset`` of the first slot, floats from one slot to the next) of a state ``[slots, n]``."""
+        _check(state, name, torch.float32)
+        if state.dim() != 2 or offset < 0 or offset + needed > state.shape[1]:
+            raise ValueError(f"{name} {tuple(state.shape)} has no room for {needed} numbers from column {offset}")
+        return state.data_ptr() + 4 * offset, state.shape[1]
+
+    def token_shift(self, h, mu, state, offset, state_slots, token_row, positions, row_start, out, keep=False):
+        n, width = h.shape
+        mixes = mu.shape[0]
+        if keep and n != row_start.shape[0]:
+            raise ValueError("the state moves on inside this kernel only in steps of one token per row")
+        _check(h, "h")
+        _check(mu, "mu", torch.float32, (mixes, width))
+        _check(out, "out", h.dtype, (mixes, n, width))
+        _check(token_row, "token_row", torch.int32, (n,))
+        _check(positions, "positions", torch.int32, (n,))
+        _check(row_start, "row_start", torch.int32)
+        _check(state_slots, "state_slots", torch.int32, (row_start.shape[0],))
+        pointer, stride = self._state_rows(state, offset, width, "state")
+        _launched(self._part_library("recurrent").lsa_token_shift(
+            _code(h), _ptr(h), _ptr(mu), mixes, pointer, stride, _ptr(state_slots), _ptr(token_row), _ptr(positions), _ptr(row_start),
+            _ptr(out), n, width, 1 if keep else 0, _stream()), "token_shift")
+
+    def token_shift_keep(self, h, state, offset, state_slots, row_start, row_len):
+        n, width = h.shape
+        rows = row_len.shape[0]
+        _check(h, "h")
+        for name, tensor in (("state_slots", state_slots), ("row_start", row_start), ("row_len", row_len)):
+            _check(tensor, name, torch.int32, (rows,))
+        pointer, stride = self._state_rows(state, offset, width, "state")
+        _launched(self._part_library("recurrent").lsa_token_shift_keep(_code(h), _ptr(h), pointer, stride, _ptr(state_slots), _ptr(row_start),
+                                                                       _ptr(row_len), rows, width, _stream()), "token_shift_keep")
+
+    def batched_linear(self, x, weights):
+        """A batched product of the library (true 32-bit on the float32 path, as every product)."""
+        return torch.bmm(x, weights.transpose(1, 2))
+
+    def tanh_(self, x):
+        _check(x, "x")
+        _launched(self._part_library("recurrent").lsa_tanh(_code(x), _ptr(x), x.numel(), _stream()), "tanh")
+
+    DECAY_MODES = ("sigmoid_root", "double_exp")
+
+    def linear_recurrence(self, q, k, v, decay, decay_bias, decay_mode, tau, bonus, q_scale, state, offset, state_slots,
+                          row_start, row_len, row_ctx, out, heads, dim, value_dim):
+        n = out.shape[0]
+        rows = row_len.shape[0]
+        if decay_mode not in self.DECAY_MODES:
+            raise ValueError(f"the recurrence kernel knows the decays {self.DECAY_MODES}, not {decay_mode!r}")
+        lib = self._part_library("recurrent")
+        if dim > lib.lsa_linear_recurrence_most_dim():
+            raise ValueError(f"the recurrence kernel takes heads of up to {lib.lsa_linear_recurrence_most_dim()} key channels, got {dim}")
+        for name, tensor, columns in (("q", q, heads * dim), ("k", k, heads * dim), ("v", v, heads * value_dim)):
+            if not tensor.is_cuda or tensor.dtype != q.dtype or tuple(tensor.shape) != (n, columns) or (n > 1 and tensor.stride(1) != 1):
+                raise ValueError(f"{name} must be a view [{n}, {columns}] of {q.dtype} on the GPU with unit stride along a row")
+        _code(q)
+        _check(decay, "decay", torch.float32, (n, heads * dim))
+        if decay_bias is not None:
+            _check(decay_bias, "decay_bias", torch.float32, (heads * dim,))
+        if bonus is not None:
+            _check(bonus, "bonus", torch.float32, (heads, dim))
+        _check(out, "out", torch.float32, (n, heads * value_dim))
+        for name, tensor in (("state_slots", state_slots), ("row_start", row_start), ("row_len", row_len), ("row_ctx", row_ctx)):
+            _check(tensor, name, torch.int32, (rows,))
+        pointer, stride = self._state_rows(state, offset, heads * dim * value_dim, "state")
+        _launched(lib.lsa_linear_recurrence(
+            _code(q), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), _ptr(decay), _ptr(decay_bias),
+            self.DECAY_MODES.index(decay_mode), float(tau), _ptr(bonus), float(q_scale), pointer, stride, _ptr(state_slots), _ptr(row_start),
+            _ptr(row_len), _ptr(row_ctx), _ptr(out), rows, heads, dim, value_dim, _stream()), "linear_recurrence")
+
+    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim):
+        n = x.shape[0]
+        _check(x, "x", torch.float32, (n, heads * value_dim))
+        _check(weight, "weight", torch.float32, (heads * value_dim if weight_per_channel else value_dim,))
+        _check(out, "out", None, (n, heads * value_dim))
+        if not gate.is_cuda or gate.dtype != out.dtype or tuple(gate.shape) != (n, heads * value_dim) or (n > 1 and gate.stride(1) != 1):
+            raise ValueError(f"gate must be a view [{n}, {heads * value_dim}] of {out.dtype} on the GPU with unit stride along a row")
+        _launched(self._part_library("recurrent").lsa_heads_norm_gate(
+            _code(out), _ptr(x), _ptr(weight), 1 if weight_per_channel else 0, float(eps), gate.data_ptr(), gate.stride(0), _ptr(out),
+            n, heads, value_dim, _stream()), "heads_norm_gate")
+
+    def scaled_sum(self, x, x_scale, y, y_scale, out):
+        _check(x, "x")
+        _check(y, "y", x.dtype, tuple(x.shape))
+        _check(out, "out", x.dtype, tuple(x.shape))
+        _launched(self._part_library("recurrent").lsa_scaled_sum(_code(x), _ptr(x), float(x_scale), _ptr(y), float(y_scale), _ptr(out),
+                                                                 x.numel(), _stream()), "scaled_sum")
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape
