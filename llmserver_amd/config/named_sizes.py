@@ -55,6 +55,29 @@ NAMED_SIZES.update({
 })
 
 
+def _barotar(width, layers, heads, kv_heads, dim, window, recurrent_heads, gla_heads, gla_dim, gla_vdim, ff, expert_ff, experts, top, groups, keep,
+             vocab=32768):
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim // 2},
+            "scale": dim ** -0.5, "softcap": 50.0}
+    parallel = {"left": left, "right": {"heads": recurrent_heads, "dim": width // recurrent_heads, "low": 64}, "left_scale": 1.0, "right_scale": 1.0}
+    gla = {"heads": gla_heads, "dim": gla_dim, "vdim": gla_vdim, "tau": 16.0, "low": 16}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}}}
+    four = [("parallel", parallel, dense), ("gla", gla, moe), ("parallel", parallel, dense), ("parallel", parallel, moe)]
+    return {"architecture": "Barotar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "layers": [{"type": kind, "mixer": dict(mixer), "mlp": dict(mlp)} for kind, mixer, mlp in (four * (-(-layers // 4)))[:layers]]}
+
+
+# Barotar at the widths of the sizes above: windowed attention of 16 (32) heads of 128 over 8 key/value heads and a window
+# of 1,024 keys beside a time mixing of as many heads of 128; a gated linear recurrence of 8 (16) heads with keys of 128 and
+# values of 256; dense feed-forwards as large as the dense decoders' beside them, and experts of the Zepolix sizes' shape
+# in groups of eight.  Three layers in four mix side by side, one in four is the linear recurrence; half the layers route.
+NAMED_SIZES.update({
+    "barotar-2k": _barotar(2048, 8, 16, 8, 128, 1024, 16, 8, 128, 256, 6 * 1408, 1408, 64, 6, 8, 4),
+    "barotar-4k": _barotar(4096, 8, 32, 8, 128, 1024, 32, 16, 128, 256, 4 * 2048, 2048, 32, 4, 4, 2),
+})
+
+
 def named_size(name: str) -> dict:
     """The entry's keys, a copy the caller may change (fewer layers, say)."""
     try:

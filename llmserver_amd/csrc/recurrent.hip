@@ -204,25 +204,52 @@ LSA_EXPORT int lsa_token_shift_keep(int code, const void* h, float* state, long 
     LSA_LAUNCH_CHECK();
 }
 
-// Key channels a wavefront takes: 8 for heads of up to 64 channels, 16 up to 256, 32 up to 512 (at most 16 wavefronts).
-LSA_EXPORT int lsa_linear_recurrence_most_dim() { return 512; }
+// Key channels a wavefront takes: 8 for heads of up to 64 channels, 16 up to 256, 32 beyond (at most 14 wavefronts: what
+// the tokens' chunk and the wavefronts' partial read-outs take of LDS then stays below the 160 KB of a compute unit).
+constexpr int MOST_DIM = 448;
+constexpr int MOST_LDS = 160 * 1024;
+
+LSA_EXPORT int lsa_linear_recurrence_most_dim() { return MOST_DIM; }
+
+static size_t recurrence_lds(int dim, int& dk, int& waves) {
+    dk = dim <= 64 ? 8 : dim <= 256 ? 16 : 32;
+    waves = (dim + dk - 1) / dk;
+    return sizeof(float) * ((size_t)3 * CHUNK * waves * dk + (size_t)CHUNK * 64 + (size_t)waves * CHUNK * 64);
+}
+
+// Once, when the library has been loaded and before any launch: lets every form of the recurrence kernel ask for more
+// dynamic LDS than the default limit.  (Not part of a launch: a launch may be recorded into a graph, and a stream
+// that is being captured must see launches only.)
+LSA_EXPORT int lsa_recurrent_prepare() {
+    hipError_t first = hipSuccess;
+#define LSA_ALLOW(T, DK, B) do { \
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_recurrence_kernel<T, DK, B>), \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, MOST_LDS); \
+        if (e != hipSuccess && first == hipSuccess) first = e; \
+    } while (0)
+#define LSA_ALLOW_ALL(T) do { LSA_ALLOW(T, 8, false); LSA_ALLOW(T, 8, true); LSA_ALLOW(T, 16, false); LSA_ALLOW(T, 16, true); \
+                              LSA_ALLOW(T, 32, false); LSA_ALLOW(T, 32, true); } while (0)
+    LSA_ALLOW_ALL(float);
+    LSA_ALLOW_ALL(bf16_t);
+#undef LSA_ALLOW_ALL
+#undef LSA_ALLOW
+    (void)hipGetLastError();
+    return (int)first;
+}
 
 LSA_EXPORT int lsa_linear_recurrence(int code, const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                                      const float* decay, const float* decay_bias, int mode, float tau, const float* bonus, float q_scale,
                                      float* state, long state_stride, const int* slots, const int* row_start, const int* row_len,
                                      const int* row_ctx, float* out, int rows, int heads, int dim, int value_dim, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (dim < 1 || dim > 512 || value_dim < 1 || heads < 1 || (mode != 0 && mode != 1) || !(tau > 0.f) || state == nullptr) return -1;
-    const int dk = dim <= 64 ? 8 : dim <= 256 ? 16 : 32;
-    const int waves = (dim + dk - 1) / dk;
-    const size_t lds = sizeof(float) * ((size_t)3 * CHUNK * waves * dk + (size_t)CHUNK * 64 + (size_t)waves * CHUNK * 64);
+    if (dim < 1 || dim > MOST_DIM || value_dim < 1 || heads < 1 || (mode != 0 && mode != 1) || !(tau > 0.f) || state == nullptr) return -1;
+    int dk, waves;
+    const size_t lds = recurrence_lds(dim, dk, waves);
+    if (lds > (size_t)MOST_LDS) return -1;
     dim3 grid(rows, heads, (value_dim + 63) / 64);
-#define LSA_LAUNCH(T, DK, B) do { \
-        if (lds > 48 * 1024) \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_recurrence_kernel<T, DK, B>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+#define LSA_LAUNCH(T, DK, B) \
         linear_recurrence_kernel<T, DK, B><<<grid, waves * 64, lds, stream>>>((const T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, \
-            decay, decay_bias, mode, 1.f / tau, bonus, q_scale, state, state_stride, slots, row_start, row_len, row_ctx, out, heads, dim, value_dim); \
-    } while (0)
+            decay, decay_bias, mode, 1.f / tau, bonus, q_scale, state, state_stride, slots, row_start, row_len, row_ctx, out, heads, dim, value_dim)
 #define LSA_BY_DK(T, B) do { if (dk == 8) LSA_LAUNCH(T, 8, B); else if (dk == 16) LSA_LAUNCH(T, 16, B); else LSA_LAUNCH(T, 32, B); } while (0)
     if (code) { if (bonus) LSA_BY_DK(bf16_t, true); else LSA_BY_DK(bf16_t, false); }
     else { if (bonus) LSA_BY_DK(float, true); else LSA_BY_DK(float, false); }

@@ -32,6 +32,7 @@ _SIGNATURES = {
     "lsa_token_shift": [c_int, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_token_shift_keep": [c_int, _P, _P, c_long, _P, _P, _P, c_int, c_int, _P],
     "lsa_linear_recurrence_most_dim": [],
+    "lsa_recurrent_prepare": [],
     "lsa_linear_recurrence": [c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, c_float, _P, c_float, _P, c_long, _P, _P, _P, _P, _P,
                               c_int, c_int, c_int, c_int, _P],
     "lsa_heads_norm_gate": [c_int, _P, _P, c_int, c_float, _P, c_long, _P, c_int, c_int, c_int, _P],

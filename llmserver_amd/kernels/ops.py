@@ -781,6 +781,10 @@ class HipOps(KernelNamespace):
         loaded = self._parts_libraries.get(name)
         if loaded is None:
             loaded = self._parts_libraries[name] = library.load(name)
+            if name == "recurrent":
+                # Once, outside any launch (a launch may be recorded into a graph): the recurrence kernel may ask for
+                # more LDS than the default limit.  If that is refused, launches that need more say so themselves.
+                loaded.lsa_recurrent_prepare()
         return loaded
 
     def embedding_norm(self, table, token_ids, weight, eps, out):

@@ -265,3 +265,34 @@ def test_gated_activation_with_the_tanh_form_of_gelu(ops, dtype):
     for which, out in zip((ops, twin), outs):
         which.swiglu(gate_up, out, activation="gelu_tanh")
     close(outs[0], outs[1], dtype, "gelu_tanh")
+
+
+def test_a_recurrence_with_heads_of_128_channels_is_recorded_into_a_graph_and_replayed(ops):
+    """Heads of 128 key channels take more LDS than a kernel gets by default; the launch must be nothing but a launch,
+    so that a captured step can hold it.  Every replay (inputs changed in place between them, eager work and
+    synchronisations in between) equals the eager result."""
+    heads, dim, vdim, n = 2, 128, 128, 40
+    make = lambda a: torch.tensor(a, dtype=torch.int32, device="cuda")
+    proj = torch.randn(n, 3 * heads * dim, device="cuda").to(torch.bfloat16)
+    q, k, v = proj[:, :heads * dim], proj[:, heads * dim:2 * heads * dim], proj[:, 2 * heads * dim:]
+    decay = torch.randn(n, heads * dim, device="cuda")
+    bonus = torch.randn(heads, dim, device="cuda")
+    state = torch.zeros(2, heads * dim * vdim, device="cuda")
+    out = torch.zeros(n, heads * vdim, device="cuda")
+    args = (q, k, v, decay, None, "double_exp", 1.0, bonus, 1.0, state, 0, make([1]), make([0]), make([n]), make([n]), out, heads, dim, vdim)
+    ops.linear_recurrence(*args)                      # (eager first, as every captured step runs)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.linear_recurrence(*args)
+    twin = TorchOps()
+    for replay in range(3):
+        proj.copy_(torch.randn(n, 3 * heads * dim, device="cuda").to(torch.bfloat16))
+        decay.copy_(torch.randn(n, heads * dim, device="cuda"))
+        graph.replay()
+        torch.cuda.synchronize()
+        want, want_state = torch.zeros_like(out), torch.zeros_like(state)
+        twin.linear_recurrence(q, k, v, decay, None, "double_exp", 1.0, bonus, 1.0, want_state, 0, make([1]), make([0]), make([n]), make([n]),
+                               want, heads, dim, vdim)
+        close(out, want, torch.float32, f"replay {replay}")
+        close(state, want_state, torch.float32, f"state after replay {replay}")
