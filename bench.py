@@ -201,6 +201,9 @@ def main() -> int:
                         help="instead of the default workload: prefill and decode of this design at a few named sizes, each beside "
                              "the dense decoder of equal width, depth and active feed-forward size")
     args = parser.parse_args()
+    if args.design in UNMEASURED_DESIGNS:
+        print(f"bench.py --design {args.design}: {UNMEASURED_DESIGNS[args.design]}", file=sys.stderr)
+        return 2
     if args.design:
         return compare_design(args)
     if args.gpus != 1:
@@ -286,6 +289,12 @@ def main() -> int:
     print(json.dumps(result), flush=True)
     return 0
 
+
+# Designs whose comparison is switched off, with the reason (the sizes stay listed below).
+UNMEASURED_DESIGNS = {
+    "barotar": "switched off: at these named sizes the first prompt steps ended with an illegal memory access on the GPU (twice), and the "
+               "kernel at fault has not been found; the tests' configurations and other model folders run (bin/trace_run, generate, benchmark.py)",
+}
 
 DESIGN_SIZES = {"zepolix": (("zepolix-2k", "dense-2k"), ("zepolix-4k", "dense-4k")),
                 "barotar": (("barotar-2k", "dense-2k"), ("barotar-4k", "dense-4k"))}

@@ -121,3 +121,16 @@ def test_greedy_generation_through_the_entry_point():
     rounded = generate(model_folder("BA"), prompts, max_new_tokens=7, dtype="bfloat16", device="cuda", block_size=8)
     same = sum(a == b for g, e in zip(rounded, expected) for a, b in zip(g, e))
     assert same >= 0.6 * sum(len(e) for e in expected), (rounded, expected)
+
+
+@pytest.mark.skip(reason="bench.py --design barotar at its named sizes (widths of 2,048 and 4,096) ended with an illegal memory access inside the "
+                         "first prompt steps on the GPU, twice; the kernel at fault has not been found by reading, so the case stays off the "
+                         "GPU (the option itself refuses to run) until it has")
+def test_the_design_option_of_bench(tmp_path):
+    """``bench.py --design barotar`` prints one JSON line with every named size beside its dense neighbour."""
+    import json
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--design", "barotar", "--layers", "2", "--steps", "4", "--warmup", "1",
+                           "--prefill-tokens", "256"], capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    record = json.loads([line for line in done.stdout.splitlines() if line.strip()][-1])
+    assert set(record["sizes"]) == {"barotar-2k", "dense-2k", "barotar-4k", "dense-4k"} and record["value"] > 0
