@@ -1,0 +1,139 @@
+"""Seeded random Barotar configurations: any order of gla and parallel layers, with dense, routed or no feed-forward;
+any number of heads and key/value heads; head, value and state sizes that are multiples of nothing, up to sizes of
+real models' heads (128 and more); rotations of nothing, a part or all of a head; windows from a few keys to more than
+any request; widths and vocabularies that are no multiple of four; decay maps of any inner size; experts in any
+grouping.  Every configuration goes through a mixed trace (pages and state slots used again): on the CPU with the
+kernels' twins, on the GPU through ``bin/trace_run`` in both types."""
+import io
+import os
+import random
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+import plain_barotar as plain
+import traces
+from helpers import random_tokens, relative_error
+from llmserver_amd.config import config_from_dict
+from llmserver_amd.engine.replay import make_runner, replay
+from llmserver_amd.weights import RandomInit, write_random_model
+from tiny_barotar import attention, config, dense, gla, moe, parallel
+from torch_ops import TorchOps
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SEEDS = list(range(8))
+FLOAT32_ERROR = 3e-5
+_MADE = {}
+
+
+def random_config(seed):
+    rng = random.Random(2000 + seed)
+    big = seed % 2 == 1                      # every other seed has heads of the sizes real models use
+    layers = []
+    for _ in range(rng.randint(1, 4)):
+        if rng.random() < 0.4:
+            dim = rng.choice([64, 128, 130]) if big else rng.randint(1, 40)
+            mixer = gla(rng.randint(1, 6), dim, rng.choice([64, 128, 256, 70]) if big else rng.randint(1, 40), rng.uniform(1.0, 20.0),
+                        low=rng.choice([None, 1, 7, 16, 64]))
+        else:
+            kv_heads = rng.randint(1, 4)
+            dim = rng.choice([64, 128, 96]) if big else rng.randint(2, 40)
+            vdim = rng.choice([dim, 64, 128]) if big else rng.randint(1, 40)
+            left = attention(kv_heads * rng.randint(1, 5), kv_heads, dim, vdim, rng.choice([1, 5, 16, 33, 64, 100, 1000]),
+                             2 * rng.randint(0, dim // 2), base=10.0 ** rng.uniform(1.5, 6.0), scale=rng.uniform(0.05, 0.5),
+                             softcap=rng.choice([1.0, 5.0, 30.0, 50.0]))
+            mixer = parallel(left, rng.randint(1, 6), rng.choice([64, 128]) if big else rng.randint(1, 40), low=rng.choice([None, 2, 16, 64]),
+                             left_scale=rng.uniform(0.3, 1.5), right_scale=rng.uniform(0.3, 1.5))
+        kind = rng.random()
+        if kind < 0.2:
+            mlp = None
+        elif kind < 0.5:
+            mlp = dense(rng.randint(3, 90))
+        else:
+            groups = rng.randint(1, 8)
+            per = rng.randint(1, 4)
+            keep = rng.randint(1, groups)
+            mlp = moe(rng.choice([32, 64, 96]) if big and rng.random() < 0.5 else rng.randint(3, 70), rng.uniform(0.5, 8.0), groups * per,
+                      rng.randint(1, min(keep * per, 6)), groups, keep)
+        layers.append((mixer, mlp))
+    width = rng.choice([64, 128, 256]) if big else rng.choice([24, 40, 50, 64, 72, 100, 134])
+    raw = config(rng.randint(30, 400), width, 10.0 ** rng.uniform(-6, -3), layers)
+    return raw, RandomInit(seed=seed, std=rng.uniform(0.08, 0.2), norm_noise=0.25, bias_std=0.4), rng.choice([4, 8, 16, 32])
+
+
+def made(seed):
+    """(config.json, folder, page size, requests, steps, exact logits per request, tensors) of a seed, made once."""
+    if seed not in _MADE:
+        raw, init, page = random_config(seed)
+        folder = tempfile.mkdtemp(prefix=f"llmserver_amd_test_br{seed}_")
+        write_random_model(config_from_dict(dict(raw)), folder, init)
+        lengths = (1, 37, 90, 5, 64, 2, 130, 18)
+        requests = {f"q{i}": random_tokens(raw["vocab"], n, 50 * seed + i) for i, n in enumerate(lengths)}
+        steps = traces.mixed(requests, seed=seed, budget_tokens=256)
+        tensors = plain.read_folder(folder)[1]
+        exact = {rid: plain.forward(raw, tensors, tokens).numpy() for rid, tokens in requests.items()}
+        _MADE[seed] = (raw, folder, page, requests, steps, exact, tensors)
+    return _MADE[seed]
+
+
+_BOUNDS = {}
+
+
+def float32_bound(seed):
+    """What a position's logits may differ by in float32, in units of their largest magnitude: three times what the plain
+    implementation itself loses when it computes in float32 (the 99th percentile over the seed's positions), and never
+    less than FLOAT32_ERROR."""
+    if seed not in _BOUNDS:
+        raw, folder, _, requests, _, exact, _ = made(seed)
+        single = plain.read_folder(folder, dtype=torch.float32)[1]
+        lost = [relative_error(row, want) for rid, tokens in requests.items()
+                for row, want in zip(plain.forward(raw, single, tokens).numpy(), exact[rid])]
+        _BOUNDS[seed] = max(FLOAT32_ERROR, 3.0 * float(np.quantile(lost, 0.99)))
+    return _BOUNDS[seed]
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_random_configurations_with_the_twins(seed, tmp_path):
+    raw, folder, page, requests, steps, exact, _ = made(seed)
+    runner = make_runner(folder, "float32", traces.peak_tokens(steps), page, device="cpu", ops=TorchOps())
+    replay(runner, traces.to_lines(steps).splitlines(), str(tmp_path), io.StringIO())
+    runner.cache.check_invariants()
+    results = traces.collect(steps, str(tmp_path), raw["vocab"])
+    assert len(results) == sum(len(t) for t in requests.values())
+    for (rid, position), logits in results.items():
+        assert relative_error(logits, exact[rid][position]) <= float32_bound(seed), f"seed {seed} {rid} {position}: {raw}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", SEEDS)
+def test_random_configurations_on_the_gpu(seed, dtype, tmp_path):
+    raw, folder, page, requests, steps, exact, tensors = made(seed)
+    print(f"random configuration {seed} {dtype}: {raw}", flush=True)
+    out = tmp_path / "out"
+    command = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
+               "--max-tokens", str(traces.peak_tokens(steps)), "--page-size", str(page)]
+    done = subprocess.run(command, input=traces.to_lines(steps), capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    results = traces.collect(steps, str(out), raw["vocab"])
+    assert len(results) == sum(len(t) for t in requests.values())
+    errors = []
+    for (rid, position), logits in results.items():
+        if dtype == "float32":
+            assert relative_error(logits, exact[rid][position]) <= float32_bound(seed), f"seed {seed} {rid} {position}: {raw}"
+        else:
+            errors.append(relative_error(logits, exact[rid][position]))
+    if errors:
+        # what the plain implementation loses on the same sequences when it rounds where 16-bit kernels round (the median held
+        # tightly, the 90th percentile loosely: a router score a rounding away from its neighbour changes a place altogether)
+        rounding = plain.rounding_to(torch.bfloat16)
+        lost = [relative_error(row, want) for rid, tokens in requests.items()
+                for row, want in zip(plain.forward(raw, tensors, tokens, r=rounding).numpy(), exact[rid])]
+        assert np.isfinite(errors).all()
+        print(f"  median {np.median(errors):.2e} / {np.median(lost):.2e}, 90th {np.quantile(errors, 0.9):.2e} / {np.quantile(lost, 0.9):.2e}", flush=True)
+        assert np.median(errors) <= 1.3 * np.median(lost), (seed, np.median(errors), np.median(lost))
+        assert np.quantile(errors, 0.9) <= 3.0 * np.quantile(lost, 0.9), (seed, np.quantile(errors, 0.9), np.quantile(lost, 0.9))
