@@ -291,10 +291,7 @@ def main() -> int:
 
 
 # Designs whose comparison is switched off, with the reason (the sizes stay listed below).
-UNMEASURED_DESIGNS = {
-    "barotar": "switched off: at these named sizes the first prompt steps ended with an illegal memory access on the GPU (twice), and the "
-               "kernel at fault has not been found; the tests' configurations and other model folders run (bin/trace_run, generate, benchmark.py)",
-}
+UNMEASURED_DESIGNS = {}
 
 DESIGN_SIZES = {"zepolix": (("zepolix-2k", "dense-2k"), ("zepolix-4k", "dense-4k")),
                 "barotar": (("barotar-2k", "dense-2k"), ("barotar-4k", "dense-4k"))}

@@ -53,7 +53,7 @@ __device__ __forceinline__ float decay_of(float z, int mode, float inv_tau) {
 }
 
 // grid (rows, heads, blocks of 64 value columns); a workgroup of NW wavefronts walks the row's tokens in order.
-// Lane = value column; wavefront w owns key channels [w * DK, (w + 1) * DK) and keeps its DK x 64 piece of the head's
+// Lane = value column; wavefront w (of up to eight) owns key channels [w * DK, (w + 1) * DK) and keeps its DK x 64 piece of the head's
 // state in registers, so the state is read once before the row's first token and written once after its last one.
 // The tokens go through LDS in chunks of CHUNK: queries (scaled), keys and decays of the head, widened and, for the
 // decays, exponentiated once per (token, channel) by whichever thread loads them; the chunk's values of this block of
@@ -65,7 +65,7 @@ __device__ __forceinline__ float decay_of(float z, int mode, float inv_tau) {
 constexpr int CHUNK = 16;
 
 template <typename T, int DK, bool BONUS>
-__global__ void linear_recurrence_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
+__global__ __launch_bounds__(512) void linear_recurrence_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
                                          const T* __restrict__ v, long v_stride, const float* __restrict__ decay,
                                          const float* __restrict__ decay_bias, int mode, float inv_tau, const float* __restrict__ bonus,
                                          float q_scale, float* state, long state_stride, const int* __restrict__ slots,
@@ -119,21 +119,31 @@ __global__ void linear_recurrence_kernel(const T* __restrict__ q, long q_stride,
         __syncthreads();
         for (int t = 0; t < n; ++t) {
             const float value = s_v[t * 64 + lane];
-            const float* tq = s_q + t * padded + channel0;
-            const float* tk = s_k + t * padded + channel0;
-            const float* td = s_d + t * padded + channel0;
-            float o = 0.f;
+            // The wavefront's channels of this token, four at a time (16-byte broadcast reads: every row of the chunk and
+            // every wavefront's first channel lie at multiples of 32 bytes), and four partial sums of the read-out, so
+            // that its chain of dependent multiply-adds is a quarter as long.
+            const float4* tq = reinterpret_cast<const float4*>(s_q + t * padded + channel0);
+            const float4* tk = reinterpret_cast<const float4*>(s_k + t * padded + channel0);
+            const float4* td = reinterpret_cast<const float4*>(s_d + t * padded + channel0);
+            float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < DK; ++i) {
-                const float kv = tk[i] * value;
-                if (BONUS) {
-                    o = __builtin_fmaf(__builtin_fmaf(u[i], kv, S[i]), tq[i], o);
-                    S[i] = __builtin_fmaf(td[i], S[i], kv);
-                } else {
-                    S[i] = __builtin_fmaf(td[i], S[i], kv);
-                    o = __builtin_fmaf(S[i], tq[i], o);
+            for (int i4 = 0; i4 < DK / 4; ++i4) {
+                const float4 q4 = tq[i4], k4 = tk[i4], d4 = td[i4];
+                const float qs[4] = {q4.x, q4.y, q4.z, q4.w}, ks[4] = {k4.x, k4.y, k4.z, k4.w}, ds[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int i = 4 * i4 + e;
+                    const float kv = ks[e] * value;
+                    if (BONUS) {
+                        o4[e] = __builtin_fmaf(__builtin_fmaf(u[i], kv, S[i]), qs[e], o4[e]);
+                        S[i] = __builtin_fmaf(ds[e], S[i], kv);
+                    } else {
+                        S[i] = __builtin_fmaf(ds[e], S[i], kv);
+                        o4[e] = __builtin_fmaf(S[i], qs[e], o4[e]);
+                    }
                 }
             }
+            const float o = (o4[0] + o4[1]) + (o4[2] + o4[3]);
             s_o[(wave * CHUNK + t) * 64 + lane] = o;
         }
         __syncthreads();
@@ -204,15 +214,15 @@ LSA_EXPORT int lsa_token_shift_keep(int code, const void* h, float* state, long 
     LSA_LAUNCH_CHECK();
 }
 
-// Key channels a wavefront takes: 8 for heads of up to 64 channels, 16 up to 256, 32 beyond (at most 14 wavefronts: what
-// the tokens' chunk and the wavefronts' partial read-outs take of LDS then stays below the 160 KB of a compute unit).
-constexpr int MOST_DIM = 448;
+// Key channels a wavefront takes: 8 for heads of up to 64 channels, 16 up to 128, 32 up to 256, 64 up to 512: at most eight
+// wavefronts a workgroup, and what the tokens' chunk and the wavefronts' partial read-outs take of LDS stays below 160 KB.
+constexpr int MOST_DIM = 512;
 constexpr int MOST_LDS = 160 * 1024;
 
 LSA_EXPORT int lsa_linear_recurrence_most_dim() { return MOST_DIM; }
 
 static size_t recurrence_lds(int dim, int& dk, int& waves) {
-    dk = dim <= 64 ? 8 : dim <= 256 ? 16 : 32;
+    dk = dim <= 64 ? 8 : dim <= 128 ? 16 : dim <= 256 ? 32 : 64;
     waves = (dim + dk - 1) / dk;
     return sizeof(float) * ((size_t)3 * CHUNK * waves * dk + (size_t)CHUNK * 64 + (size_t)waves * CHUNK * 64);
 }
@@ -228,7 +238,7 @@ LSA_EXPORT int lsa_recurrent_prepare() {
         if (e != hipSuccess && first == hipSuccess) first = e; \
     } while (0)
 #define LSA_ALLOW_ALL(T) do { LSA_ALLOW(T, 8, false); LSA_ALLOW(T, 8, true); LSA_ALLOW(T, 16, false); LSA_ALLOW(T, 16, true); \
-                              LSA_ALLOW(T, 32, false); LSA_ALLOW(T, 32, true); } while (0)
+                              LSA_ALLOW(T, 32, false); LSA_ALLOW(T, 32, true); LSA_ALLOW(T, 64, false); LSA_ALLOW(T, 64, true); } while (0)
     LSA_ALLOW_ALL(float);
     LSA_ALLOW_ALL(bf16_t);
 #undef LSA_ALLOW_ALL
@@ -250,7 +260,8 @@ LSA_EXPORT int lsa_linear_recurrence(int code, const void* q, long q_stride, con
 #define LSA_LAUNCH(T, DK, B) \
         linear_recurrence_kernel<T, DK, B><<<grid, waves * 64, lds, stream>>>((const T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, \
             decay, decay_bias, mode, 1.f / tau, bonus, q_scale, state, state_stride, slots, row_start, row_len, row_ctx, out, heads, dim, value_dim)
-#define LSA_BY_DK(T, B) do { if (dk == 8) LSA_LAUNCH(T, 8, B); else if (dk == 16) LSA_LAUNCH(T, 16, B); else LSA_LAUNCH(T, 32, B); } while (0)
+#define LSA_BY_DK(T, B) do { if (dk == 8) LSA_LAUNCH(T, 8, B); else if (dk == 16) LSA_LAUNCH(T, 16, B); else if (dk == 32) LSA_LAUNCH(T, 32, B); \
+                             else LSA_LAUNCH(T, 64, B); } while (0)
     if (code) { if (bonus) LSA_BY_DK(bf16_t, true); else LSA_BY_DK(bf16_t, false); }
     else { if (bonus) LSA_BY_DK(float, true); else LSA_BY_DK(float, false); }
 #undef LSA_BY_DK

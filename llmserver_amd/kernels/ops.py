@@ -1096,8 +1096,14 @@ class HipOps(KernelNamespace):
                                                                        _ptr(row_len), rows, width, _stream()), "token_shift_keep")
 
     def batched_linear(self, x, weights):
-        """A batched product of the library (true 32-bit on the float32 path, as every product)."""
-        return torch.bmm(x, weights.transpose(1, 2))
+        """One product per batch entry, each the way :meth:`linear` goes for its size (the few-row kernels while decoding,
+        the library for portions).  Not the library's batched product: ``torch.bmm`` of ``[4, T, 2048]`` with the transposed
+        view of ``[4, 2048, 2048]`` in bfloat16 ended with an illegal memory access on an MI355X (512 and 2,048 rows)."""
+        batch, rows, _ = x.shape
+        out = torch.empty((batch, rows, weights.shape[1]), device=x.device, dtype=x.dtype)
+        for index in range(batch):
+            self.linear(x[index], weights[index], out=out[index])
+        return out
 
     def tanh_(self, x):
         _check(x, "x")

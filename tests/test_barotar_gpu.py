@@ -123,9 +123,6 @@ def test_greedy_generation_through_the_entry_point():
     assert same >= 0.6 * sum(len(e) for e in expected), (rounded, expected)
 
 
-@pytest.mark.skip(reason="bench.py --design barotar at its named sizes (widths of 2,048 and 4,096) ended with an illegal memory access inside the "
-                         "first prompt steps on the GPU, twice; the kernel at fault has not been found by reading, so the case stays off the "
-                         "GPU (the option itself refuses to run) until it has")
 def test_the_design_option_of_bench(tmp_path):
     """``bench.py --design barotar`` prints one JSON line with every named size beside its dense neighbour."""
     import json
