@@ -98,23 +98,34 @@ __global__ __launch_bounds__(512) void linear_recurrence_kernel(const T* __restr
     for (int t0 = 0; t0 < count; t0 += CHUNK) {
         const int n = min(CHUNK, count - t0);
         __syncthreads();                                 // the chunk before has been read out of LDS
-        for (int i = threadIdx.x; i < n * padded; i += blockDim.x) {
+        // A thread stages PER numbers of each kind (CHUNK * padded = PER * blockDim.x): all their loads first, so that they are
+        // in flight together, then the decays' exponentials and the stores.
+        constexpr int PER = CHUNK * DK / 64;
+        float raw_q[PER], raw_k[PER], raw_z[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
             const int t = i / padded, c = i - t * padded;
-            const size_t token = (size_t)(start + t0 + t);
-            float qv = 0.f, kv = 0.f, dv = 1.f;
-            if (c < dim) {
-                qv = (float)q[token * q_stride + key_column + c] * q_scale;
-                kv = (float)k[token * k_stride + key_column + c];
-                const float z = decay[token * (size_t)heads * dim + key_column + c] + (decay_bias ? decay_bias[key_column + c] : 0.f);
-                dv = decay_of(z, mode, inv_tau);
+            raw_q[j] = 0.f; raw_k[j] = 0.f; raw_z[j] = 0.f;
+            if (t < n && c < dim) {
+                const size_t token = (size_t)(start + t0 + t);
+                raw_q[j] = (float)q[token * q_stride + key_column + c];
+                raw_k[j] = (float)k[token * k_stride + key_column + c];
+                raw_z[j] = decay[token * (size_t)heads * dim + key_column + c] + (decay_bias ? decay_bias[key_column + c] : 0.f);
             }
-            s_q[i] = qv;
-            s_k[i] = kv;
-            s_d[i] = dv;
         }
         for (int i = threadIdx.x; i < n * 64; i += blockDim.x) {
             const int t = i >> 6, c = column0 + (i & 63);
             s_v[i] = c < value_dim ? (float)v[(size_t)(start + t0 + t) * v_stride + (size_t)head * value_dim + c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            const int t = i / padded, c = i - t * padded;
+            if (t >= n) continue;
+            s_q[i] = raw_q[j] * q_scale;
+            s_k[i] = raw_k[j];
+            s_d[i] = c < dim ? decay_of(raw_z[j], mode, inv_tau) : 1.f;
         }
         __syncthreads();
         for (int t = 0; t < n; ++t) {
