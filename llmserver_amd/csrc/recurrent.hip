@@ -52,6 +52,36 @@ __device__ __forceinline__ float decay_of(float z, int mode, float inv_tau) {
     return expf(-expf(z));
 }
 
+// One token of one wavefront's DK channels: the state's update and the channels' part of the read-out.  The channels come
+// from LDS four at a time (16-byte broadcast reads: every row of a chunk and every wavefront's first channel lie at
+// multiples of 32 bytes); four partial sums of the read-out make its chain of dependent multiply-adds a quarter as long.
+template <int DK, bool BONUS>
+__device__ __forceinline__ float recurrence_token(float (&S)[DK], const float (&u)[DK], const float* q_row, const float* k_row,
+                                                  const float* d_row, float value) {
+    const float4* tq = reinterpret_cast<const float4*>(q_row);
+    const float4* tk = reinterpret_cast<const float4*>(k_row);
+    const float4* td = reinterpret_cast<const float4*>(d_row);
+    float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i4 = 0; i4 < DK / 4; ++i4) {
+        const float4 q4 = tq[i4], k4 = tk[i4], d4 = td[i4];
+        const float qs[4] = {q4.x, q4.y, q4.z, q4.w}, ks[4] = {k4.x, k4.y, k4.z, k4.w}, ds[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int i = 4 * i4 + e;
+            const float kv = ks[e] * value;
+            if (BONUS) {
+                o4[e] = __builtin_fmaf(__builtin_fmaf(u[i], kv, S[i]), qs[e], o4[e]);
+                S[i] = __builtin_fmaf(ds[e], S[i], kv);
+            } else {
+                S[i] = __builtin_fmaf(ds[e], S[i], kv);
+                o4[e] = __builtin_fmaf(S[i], qs[e], o4[e]);
+            }
+        }
+    }
+    return (o4[0] + o4[1]) + (o4[2] + o4[3]);
+}
+
 // grid (rows, heads, blocks of 64 value columns); a workgroup of NW wavefronts walks the row's tokens in order.
 // Lane = value column; wavefront w (of up to eight) owns key channels [w * DK, (w + 1) * DK) and keeps its DK x 64 piece of the head's
 // state in registers, so the state is read once before the row's first token and written once after its last one.
@@ -128,34 +158,21 @@ __global__ __launch_bounds__(512) void linear_recurrence_kernel(const T* __restr
             s_d[i] = c < dim ? decay_of(raw_z[j], mode, inv_tau) : 1.f;
         }
         __syncthreads();
-        for (int t = 0; t < n; ++t) {
-            const float value = s_v[t * 64 + lane];
-            // The wavefront's channels of this token, four at a time (16-byte broadcast reads: every row of the chunk and
-            // every wavefront's first channel lie at multiples of 32 bytes), and four partial sums of the read-out, so
-            // that its chain of dependent multiply-adds is a quarter as long.
-            const float4* tq = reinterpret_cast<const float4*>(s_q + t * padded + channel0);
-            const float4* tk = reinterpret_cast<const float4*>(s_k + t * padded + channel0);
-            const float4* td = reinterpret_cast<const float4*>(s_d + t * padded + channel0);
-            float o4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (DK <= 16 && n == CHUNK) {
+            // A whole chunk: the tokens' steps unrolled, their read-outs kept in registers and stored behind the last one, so
+            // that no store to LDS stands between one token's loads and the next one's and the loads can run ahead.  (With
+            // more channels a wavefront the state alone fills the registers, and running ahead would spill.)
+            float kept[CHUNK];
 #pragma unroll
-            for (int i4 = 0; i4 < DK / 4; ++i4) {
-                const float4 q4 = tq[i4], k4 = tk[i4], d4 = td[i4];
-                const float qs[4] = {q4.x, q4.y, q4.z, q4.w}, ks[4] = {k4.x, k4.y, k4.z, k4.w}, ds[4] = {d4.x, d4.y, d4.z, d4.w};
+            for (int t = 0; t < CHUNK; ++t)
+                kept[t] = recurrence_token<DK, BONUS>(S, u, s_q + t * padded + channel0, s_k + t * padded + channel0,
+                                                      s_d + t * padded + channel0, s_v[t * 64 + lane]);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = 4 * i4 + e;
-                    const float kv = ks[e] * value;
-                    if (BONUS) {
-                        o4[e] = __builtin_fmaf(__builtin_fmaf(u[i], kv, S[i]), qs[e], o4[e]);
-                        S[i] = __builtin_fmaf(ds[e], S[i], kv);
-                    } else {
-                        S[i] = __builtin_fmaf(ds[e], S[i], kv);
-                        o4[e] = __builtin_fmaf(S[i], qs[e], o4[e]);
-                    }
-                }
-            }
-            const float o = (o4[0] + o4[1]) + (o4[2] + o4[3]);
-            s_o[(wave * CHUNK + t) * 64 + lane] = o;
+            for (int t = 0; t < CHUNK; ++t) s_o[(wave * CHUNK + t) * 64 + lane] = kept[t];
+        } else {
+            for (int t = 0; t < n; ++t)
+                s_o[(wave * CHUNK + t) * 64 + lane] = recurrence_token<DK, BONUS>(S, u, s_q + t * padded + channel0, s_k + t * padded + channel0,
+                                                                                  s_d + t * padded + channel0, s_v[t * 64 + lane]);
         }
         __syncthreads();
         for (int i = threadIdx.x; i < n * 64; i += blockDim.x) {
