@@ -7,8 +7,9 @@
 using namespace lsa;
 
 // out[m][t] = h[t] + (before[t] - h[t]) * mu[m], before[t] = the row of the token before t in its request: a row of this
-// step, the request's state for a row's first token, zeros at position 0.  One workgroup per token.  keep (only in
-// steps of one token per row, where a row's state is one workgroup's): the state becomes this token's row.
+// step, the request's state for a row's first token, zeros at position 0.  grid (tokens, blocks of 256 columns): a thread
+// has one column of one token, so its two loads are the only ones it waits for.  keep (only in steps of one token per
+// row, where a column of a row's state is one thread's): the state becomes this token's row.
 template <typename T>
 __global__ __launch_bounds__(256) void token_shift_kernel(const T* __restrict__ h, const float* __restrict__ mu, int mixes,
                                                           float* state, long state_stride, const int* __restrict__ slots,
@@ -19,7 +20,7 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const T* __restrict__ 
     const int row = token_row[t];
     const bool first_of_sequence = positions[t] == 0, first_of_row = t == row_start[row];
     float* mine = state + (size_t)slots[row] * state_stride;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
         const float own = (float)h[(size_t)t * width + c];
         float before = 0.f;
         if (!first_of_sequence) before = first_of_row ? mine[c] : (float)h[(size_t)(t - 1) * width + c];
@@ -226,7 +227,8 @@ LSA_EXPORT int lsa_token_shift(int code, const void* h, const float* mu, int mix
                                int keep, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (mixes < 1 || state == nullptr || slots == nullptr) return -1;
-#define LSA_LAUNCH(T) token_shift_kernel<T><<<n_tokens, 256, 0, stream>>>((const T*)h, mu, mixes, state, state_stride, slots, token_row, positions, \
+    const dim3 grid(n_tokens, (width + 255) / 256);
+#define LSA_LAUNCH(T) token_shift_kernel<T><<<grid, 256, 0, stream>>>((const T*)h, mu, mixes, state, state_stride, slots, token_row, positions, \
         row_start, (T*)out, n_tokens, width, keep)
     if (code) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
 #undef LSA_LAUNCH
